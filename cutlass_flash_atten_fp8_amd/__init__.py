@@ -1,0 +1,166 @@
+"""FP8 flash-attention forward for AMD MI355X (gfx950).
+
+Host-side mirror of the reference's operator interface (weishengying/cutlass_flash_atten_fp8):
+
+    from attention_cutlass_fp8 import flash_attention_v2_cutlass       # reference test.py:3
+    o = flash_attention_v2_cutlass(q, k, v, is_causal, softmax_scale)[0]
+
+`attention_cutlass_fp8` is the compiled PyTorch binding (csrc/attention_api.cpp); importing this package
+registers it under that top-level name.  `flash_attention_v2_cutlass` below is the same operator driven
+from Python through the C ABI of libfa8.so (include/fa8_api.h) with ctypes; both end in the same HIP
+kernels.  There is no CPU or PyTorch fallback: if libfa8.so is missing, importing the operator raises.
+"""
+import ctypes
+import importlib.util
+import os
+import sys
+import sysconfig
+
+_PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+LIBFA8_PATH = os.path.join(_PKG_DIR, "libfa8.so")
+_EXT_NAME = "attention_cutlass_fp8"
+EXT_PATH = os.path.join(_PKG_DIR, _EXT_NAME + sysconfig.get_config_var("EXT_SUFFIX"))
+
+# codes of include/fa8_api.h
+FA8_DTYPE_E4M3, FA8_DTYPE_E5M2 = 0, 1
+FA8_OUT_FP16, FA8_OUT_E4M3 = 0, 1
+FA8_V_ROWS, FA8_V_TRANSPOSED = 0, 1
+FA8_QUERY_VERSION, FA8_QUERY_KV_BLOCK, FA8_QUERY_Q_BLOCK, FA8_QUERY_KV_ASCENDING, FA8_QUERY_THREADS = range(5)
+FA8_EXPORTS = ("fa8_fwd_validate", "fa8_fwd", "fa8_query", "fa8_error_string")
+
+
+class Fa8FwdParams(ctypes.Structure):
+    """struct Fa8FwdParams of include/fa8_api.h."""
+    _fields_ = [
+        ("q", ctypes.c_void_p), ("k", ctypes.c_void_p), ("v", ctypes.c_void_p), ("o", ctypes.c_void_p),
+        ("batch", ctypes.c_int32), ("heads", ctypes.c_int32), ("seqlen_q", ctypes.c_int32),
+        ("seqlen_k", ctypes.c_int32), ("head_dim", ctypes.c_int32), ("is_causal", ctypes.c_int32),
+        ("in_dtype", ctypes.c_int32), ("out_dtype", ctypes.c_int32), ("v_layout", ctypes.c_int32),
+        ("softmax_scale", ctypes.c_float),
+        ("q_batch_stride", ctypes.c_int64), ("q_head_stride", ctypes.c_int64), ("q_row_stride", ctypes.c_int64),
+        ("k_batch_stride", ctypes.c_int64), ("k_head_stride", ctypes.c_int64), ("k_row_stride", ctypes.c_int64),
+        ("v_batch_stride", ctypes.c_int64), ("v_head_stride", ctypes.c_int64), ("v_row_stride", ctypes.c_int64),
+        ("o_batch_stride", ctypes.c_int64), ("o_head_stride", ctypes.c_int64), ("o_row_stride", ctypes.c_int64),
+    ]
+
+
+_lib = None
+
+
+def lib():
+    """The loaded libfa8.so with typed entry points.  Raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIBFA8_PATH):
+            raise ImportError(
+                f"{LIBFA8_PATH} is missing: build it with `python -m cutlass_flash_atten_fp8_amd.build` "
+                "(there is no CPU or PyTorch fallback for the attention kernels)")
+        L = ctypes.CDLL(LIBFA8_PATH)
+        L.fa8_fwd_validate.restype = ctypes.c_int
+        L.fa8_fwd_validate.argtypes = [ctypes.POINTER(Fa8FwdParams)]
+        L.fa8_fwd.restype = ctypes.c_int
+        L.fa8_fwd.argtypes = [ctypes.POINTER(Fa8FwdParams), ctypes.c_void_p]
+        L.fa8_query.restype = ctypes.c_int
+        L.fa8_query.argtypes = [ctypes.c_int]
+        L.fa8_error_string.restype = ctypes.c_char_p
+        L.fa8_error_string.argtypes = [ctypes.c_int]
+        _lib = L
+    return _lib
+
+
+def error_string(code):
+    return lib().fa8_error_string(int(code)).decode()
+
+
+def query(what):
+    return int(lib().fa8_query(int(what)))
+
+
+def load_extension():
+    """Import the compiled binding and register it as the top-level module `attention_cutlass_fp8`."""
+    if _EXT_NAME in sys.modules:
+        return sys.modules[_EXT_NAME]
+    if not os.path.exists(EXT_PATH):
+        raise ImportError(f"{EXT_PATH} is missing: build it with `python -m cutlass_flash_atten_fp8_amd.build`")
+    import torch  # noqa: F401  (the binding links against libtorch)
+    spec = importlib.util.spec_from_file_location(_EXT_NAME, EXT_PATH)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    sys.modules[_EXT_NAME] = mod
+    return mod
+
+
+def make_params(q, k, v, o, is_causal, softmax_scale, v_transposed=False):
+    """Fill Fa8FwdParams from torch tensors (any device: only shapes, strides and pointers are read)."""
+    import torch
+    in_codes = {torch.float8_e4m3fn: FA8_DTYPE_E4M3, torch.float8_e5m2: FA8_DTYPE_E5M2}
+    out_codes = {torch.float16: FA8_OUT_FP16, torch.float8_e4m3fn: FA8_OUT_E4M3}
+    if q.dtype not in in_codes:
+        raise RuntimeError(f"q must be torch.float8_e4m3fn or torch.float8_e5m2 (OCP fp8), got {q.dtype}")
+    if k.dtype != q.dtype or v.dtype != q.dtype:
+        raise RuntimeError("q, k and v must have the same dtype")
+    if o.dtype not in out_codes:
+        raise RuntimeError("out_dtype must be torch.float16 or torch.float8_e4m3fn")
+    for name, t in (("q", q), ("k", k), ("v", v), ("o", o)):
+        if t.dim() != 4:
+            raise RuntimeError(f"{name} must be 4-dimensional [batch, heads, seqlen, head_dim], got {t.dim()} dims")
+        if t.stride(3) != 1:
+            raise RuntimeError(f"the last dimension of {name} must be contiguous")
+    p = Fa8FwdParams()
+    p.q, p.k, p.v, p.o = q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr()
+    p.batch, p.heads, p.seqlen_q, p.head_dim = q.shape
+    p.seqlen_k = k.shape[2]
+    p.is_causal = int(bool(is_causal))
+    p.in_dtype = in_codes[q.dtype]
+    p.out_dtype = out_codes[o.dtype]
+    p.v_layout = FA8_V_TRANSPOSED if v_transposed else FA8_V_ROWS
+    p.softmax_scale = float(softmax_scale)
+    for name, t in (("q", q), ("k", k), ("v", v), ("o", o)):
+        setattr(p, name + "_batch_stride", t.stride(0))
+        setattr(p, name + "_head_stride", t.stride(1))
+        setattr(p, name + "_row_stride", t.stride(2))
+    return p
+
+
+def flash_attention_v2_cutlass(q, k, v, is_causal, softmax_scale, *, v_transposed=False, out_dtype=None):
+    """The reference operator (reference csrc/flash_attention.cu:639-668) through the C ABI.
+
+    q, k: fp8 [B,H,N,d] on the GPU; v: [B,H,N,d] (or [B,H,d,N] with v_transposed=True, as the reference
+    requires of its caller, test.py:71).  Returns [O], O fp16 [B,H,N,d] (out_dtype=torch.float8_e4m3fn
+    gives the reference's fp8 O).  Runs on torch's current stream without synchronising.  Raises
+    RuntimeError on bad arguments, like the reference's TORCH_CHECKs (include/attention_api.cuh:12-18).
+    """
+    import torch
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        if not t.is_cuda:
+            raise RuntimeError(f"{name} must be a GPU tensor")
+        if not t.is_contiguous():
+            raise RuntimeError(f"{name} must be contiguous")
+        if t.dim() != 4:
+            raise RuntimeError(f"{name} must be 4-dimensional [batch, heads, seqlen, head_dim], got {t.dim()} dims")
+    B, H, Nq, D = q.shape
+    Nk = k.shape[2]
+    if tuple(k.shape) != (B, H, Nk, D):
+        raise RuntimeError(f"k must be [{B}, {H}, seqlen_k, {D}], got {tuple(k.shape)}")
+    want_v = (B, H, D, Nk) if v_transposed else (B, H, Nk, D)
+    if tuple(v.shape) != want_v:
+        raise RuntimeError(f"v must be {list(want_v)}, got {tuple(v.shape)}")
+    if k.device != q.device or v.device != q.device:
+        raise RuntimeError("q, k and v must be on the same device")
+    o = torch.empty((B, H, Nq, D), dtype=out_dtype or torch.float16, device=q.device)
+    p = make_params(q, k, v, o, is_causal, softmax_scale, v_transposed)
+    with torch.cuda.device(q.device):
+        stream = torch.cuda.current_stream(q.device).cuda_stream
+        rc = lib().fa8_fwd(ctypes.byref(p), ctypes.c_void_p(stream))
+    if rc != 0:
+        raise RuntimeError(f"flash_attention_v2_cutlass: {error_string(rc)} (code {rc})")
+    return [o]
+
+
+# Make `from attention_cutlass_fp8 import flash_attention_v2_cutlass` work once this package is imported
+# (only when the binding has been built; the ctypes operator above does not need it).
+if os.path.exists(EXT_PATH) and os.path.exists(LIBFA8_PATH):
+    try:
+        load_extension()
+    except Exception as _e:  # pragma: no cover - reported on first explicit load_extension()
+        _EXT_IMPORT_ERROR = _e

@@ -1,0 +1,69 @@
+"""Builds the native code of this package in-tree.
+
+  libfa8.so                      hipcc --offload-arch=gfx950: kernels + C ABI (include/fa8_api.h)
+  attention_cutlass_fp8.*.so     g++ host-only PyTorch binding that calls libfa8.so
+
+Run as `python -m cutlass_flash_atten_fp8_amd.build` or through __graft_entry__.build().
+"""
+import os
+import subprocess
+import sys
+import sysconfig
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(PKG_DIR, "csrc")
+INCLUDE = os.path.join(os.path.dirname(PKG_DIR), "include")
+ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
+LIBFA8 = os.path.join(PKG_DIR, "libfa8.so")
+EXT_NAME = "attention_cutlass_fp8"
+EXT_PATH = os.path.join(PKG_DIR, EXT_NAME + sysconfig.get_config_var("EXT_SUFFIX"))
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    # never let the compiler form packed fp32 VALU ops
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+
+def _run(cmd):
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        sys.stderr.write(r.stdout + r.stderr)
+        raise RuntimeError("command failed: " + " ".join(cmd))
+    return r
+
+
+def build_libfa8():
+    cmd = [os.path.join(ROCM, "bin", "hipcc")] + HIPCC_FLAGS + ["-I", INCLUDE, "-o", LIBFA8,
+                                                               os.path.join(CSRC, "fa8_fwd_gfx950.hip")]
+    _run(cmd)
+    return LIBFA8
+
+
+def build_binding():
+    import torch
+    from torch.utils import cpp_extension
+    torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    inc = cpp_extension.include_paths()
+    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-w",
+           "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", "-DTORCH_EXTENSION_NAME=" + EXT_NAME,
+           "-DTORCH_API_INCLUDE_EXTENSION_H", "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI),
+           "-I", INCLUDE, "-I", os.path.join(ROCM, "include"), "-I", sysconfig.get_paths()["include"]]
+    for i in inc:
+        cmd += ["-I", i]
+    cmd += [os.path.join(CSRC, "attention_api.cpp"), "-o", EXT_PATH,
+            "-L", PKG_DIR, "-l:libfa8.so", "-L", torch_lib, "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch_hip",
+            "-ltorch", "-ltorch_python", "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + torch_lib]
+    _run(cmd)
+    return EXT_PATH
+
+
+def build_all():
+    build_libfa8()
+    build_binding()
+    return LIBFA8, EXT_PATH
+
+
+if __name__ == "__main__":
+    for p in build_all():
+        print("built", p)

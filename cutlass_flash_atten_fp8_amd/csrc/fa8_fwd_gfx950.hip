@@ -1,0 +1,473 @@
+// FP8 flash-attention forward for gfx950 (MI355X): kernels and the C-ABI launcher (libfa8.so).
+//
+// One workgroup = 4 wavefronts = 128 query rows of one (batch, head); every wavefront owns 32 query
+// rows and the whole head dimension.  KV is walked in ascending blocks of 64 rows, the block size
+// the reference instantiates (kBlockM = kBlockN = 64, reference csrc/flash_attention.cu:624), so the
+// running max that P is quantised against evolves exactly as in the reference loop
+// (csrc/flash_attention.cu:468-534).
+//
+// Formulation (different from the reference, which computes S = Q K^T with m16n8k32 atoms,
+// csrc/mma_sm89.hpp:10-35):
+//   * S^T = K Q^T with v_mfma_f32_32x32x64_f8f6f4 (A = K tile from LDS, B = Q held in registers).
+//     In the 32x32 accumulator layout a lane owns ONE query column and 16 kv rows, so the online
+//     softmax row max / row sum (reference csrc/utils.h:22-98 quad butterflies) are in-register
+//     reductions plus one v_permlane32_swap.
+//   * O^T = V^T P^T with the same instruction (A = V^T, B = P^T).  The fp32 -> fp8 P registers of a
+//     lane already are a valid B operand when the K tile rows are stored in LDS in a permuted order
+//     (kv_of_lds_row below); this replaces the reference's accumulator-to-A-operand reshuffle
+//     (csrc/reg2reg.h:31-96).  V^T fragments come from the row-major V tile in LDS through the
+//     transposing LDS read ds_read_b64_tr_b8, so V is consumed as [B,H,N,d] with no extra pass.
+//   * K and V tiles go HBM -> LDS with global_load_lds_dwordx4 (no register staging), double
+//     buffered, one barrier per KV block; 16-byte chunks are XOR-swizzled against bank conflicts,
+//     the swizzle being applied on the global-address side of the copy.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdint>
+
+#include "fa8_api.h"
+
+namespace {
+
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+
+#define LDS_PTR(T, p) ((__attribute__((address_space(3))) T*)(p))
+#define GLOBAL_PTR(T, p) ((__attribute__((address_space(1))) T*)(p))
+
+constexpr int kQBlock = 128;   // query rows per workgroup
+constexpr int kQWave = 32;     // query rows per wavefront
+constexpr int kKvBlock = 64;   // kv rows per online-softmax step
+constexpr int kThreads = 256;  // 4 wavefronts
+constexpr int kVersion = 1;
+
+struct KernelArgs {
+  const uint8_t* q;
+  const uint8_t* k;
+  const uint8_t* v;
+  void* o;
+  int heads, seqlen_q, seqlen_k, n_qblocks, bh_total;
+  float scale_log2;  // softmax_scale * log2(e)
+  long long q_bs, q_hs, q_rs;
+  long long k_bs, k_hs, k_rs;
+  long long v_bs, v_hs, v_rs;
+  long long o_bs, o_hs, o_rs;
+};
+
+// LDS row r (0..63) of a K tile holds kv row kv_of_lds_row(r) of the block.  With this order the 16
+// accumulator registers a lane gets from S^T sub-tile t (rows 8a+4h+b of the 32x32 result, h = lane/32)
+// are kv rows 32h+16t+(4a+b): exactly the bytes 16t..16t+15 of the lane's B operand in the PV MFMA.
+__device__ __forceinline__ int kv_of_lds_row(int r) {
+  const int t = r >> 5, a = (r >> 3) & 3, h = (r >> 2) & 1, b = r & 3;
+  return 32 * h + 16 * t + 4 * a + b;
+}
+
+// Swizzle: a tile is an array of 128-byte lines of eight 16-byte chunks.  For D = 128 a line is a
+// row; for D = 64 a line is two rows.  chunk_slot() gives the chunk position inside the line.
+template <int D, bool IS_V>
+__device__ __forceinline__ int tile_offset(int row, int chunk) {
+  if constexpr (D == 128) {
+    const int key = IS_V ? (row & 7) : ((row & 7) ^ ((row >> 3) & 1));
+    return row * 128 + ((chunk ^ key) << 4);
+  } else {
+    const int line = row >> 1;
+    const int key = IS_V ? (line & 3) : ((line & 3) ^ ((line >> 2) & 1));
+    return line * 128 + ((((row & 1) << 2) | (chunk ^ key)) << 4);
+  }
+}
+
+// Inverse of tile_offset for the copy engine: which (row, chunk) lives at 16-byte slot `slot`.
+template <int D, bool IS_V>
+__device__ __forceinline__ void tile_slot_decode(int slot, int& row, int& chunk) {
+  if constexpr (D == 128) {
+    row = slot >> 3;
+    const int key = IS_V ? (row & 7) : ((row & 7) ^ ((row >> 3) & 1));
+    chunk = (slot & 7) ^ key;
+  } else {
+    const int line = slot >> 3, w = slot & 7;
+    const int key = IS_V ? (line & 3) : ((line & 3) ^ ((line >> 2) & 1));
+    row = line * 2 + (w >> 2);
+    chunk = (w & 3) ^ key;
+  }
+}
+
+// v_permlane32_swap exchanges lanes 32-63 of its first operand with lanes 0-31 of its second.  Fed the same
+// value x twice it returns {x of the low half-lane, x of the high half-lane} in every lane of a query.
+typedef unsigned v2u __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float lane32_max(float x) {
+  const v2u r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float lane32_sum(float x) {
+  const v2u r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+template <bool E5M2>
+__device__ __forceinline__ v16f mfma_fp8(const v8i& a, const v8i& b, const v16f& c) {
+  if constexpr (E5M2)
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 1, 1, 0, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
+}
+
+template <bool E5M2>
+__device__ __forceinline__ int pack4_fp8(float a, float b, float c, float d) {
+  int r = 0;
+  if constexpr (E5M2) {
+    r = __builtin_amdgcn_cvt_pk_bf8_f32(a, b, r, false);
+    r = __builtin_amdgcn_cvt_pk_bf8_f32(c, d, r, true);
+  } else {
+    r = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, r, false);
+    r = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, r, true);
+  }
+  return r;
+}
+
+// Workgroup id -> (batch*head, q block).  Workgroups are dealt to the 8 XCDs round-robin by id; when
+// batch*heads is a multiple of 8 all q blocks of one head are kept on one XCD so its K/V stay in that
+// XCD's L2.  Causal problems start with the longest (last) q blocks.
+template <bool CAUSAL>
+__device__ __forceinline__ void decode_block(const KernelArgs& a, int id, int& bh, int& qb) {
+  int qi;
+  if ((a.bh_total & 7) == 0) {
+    const int xcd = id & 7, s = id >> 3;
+    bh = (s / a.n_qblocks) * 8 + xcd;
+    qi = s % a.n_qblocks;
+  } else {
+    bh = id / a.n_qblocks;
+    qi = id % a.n_qblocks;
+  }
+  qb = CAUSAL ? (a.n_qblocks - 1 - qi) : qi;
+}
+
+template <int D, bool CAUSAL, bool E5M2, int OUT>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3))) void fa8_fwd_kernel(
+    const KernelArgs a) {
+  constexpr int kTileBytes = kKvBlock * D;      // one K or V tile
+  constexpr int kStageBytes = 2 * kTileBytes;   // K tile then V tile
+  constexpr int kPasses = kTileBytes / (kThreads * 16);
+  constexpr int kKSteps = D / 64;  // MFMA k-steps over the head dim for S^T
+  constexpr int kMTiles = D / 32;  // 32-row tiles of O^T
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int qn = lane & 31, h = lane >> 5;
+
+  int bh, qb;
+  decode_block<CAUSAL>(a, blockIdx.x, bh, qb);
+  const int b = bh / a.heads, hd = bh - b * a.heads;
+  const int q0 = qb * kQBlock;
+  const int q_wave0 = q0 + wave * kQWave;
+  const int q_row = q_wave0 + qn;  // this lane's query row
+  const uint8_t* qp = a.q + b * a.q_bs + hd * a.q_hs;
+  const uint8_t* kp = a.k + b * a.k_bs + hd * a.k_hs;
+  const uint8_t* vp = a.v + b * a.v_bs + hd * a.v_hs;
+  const float c = a.scale_log2;
+
+  // ---- Q fragment (B operand of S^T = K Q^T): row q_row, bytes [64ks + 32h, +32) ----
+  v8i qf[kKSteps];
+  {
+    const int qr = min(q_row, a.seqlen_q - 1);
+    const uint8_t* src = qp + (long long)qr * a.q_rs + 32 * h;
+#pragma unroll
+    for (int ks = 0; ks < kKSteps; ++ks) {
+      const v4i lo = *(const v4i*)(src + 64 * ks);
+      const v4i hi = *(const v4i*)(src + 64 * ks + 16);
+      qf[ks] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    }
+  }
+
+  // ---- per-lane constants of the HBM -> LDS copy ----
+  // In pass p wavefront w fills LDS bytes [(4p+w)*1024, +1024) of the tile, lane l the 16 bytes at +16l.
+  int k_row[kPasses], k_col[kPasses], v_row[kPasses], v_col[kPasses];
+#pragma unroll
+  for (int p = 0; p < kPasses; ++p) {
+    const int slot = (p * 4 + wave) * 64 + lane;
+    int r, ch;
+    tile_slot_decode<D, false>(slot, r, ch);
+    k_row[p] = kv_of_lds_row(r);
+    k_col[p] = ch * 16;
+    tile_slot_decode<D, true>(slot, r, ch);
+    v_row[p] = r;
+    v_col[p] = ch * 16;
+  }
+  const int kv_last = a.seqlen_k - 1;
+  auto issue_tile = [&](int j, int stage) {
+    uint8_t* kb = smem + stage * kStageBytes;
+    uint8_t* vb = kb + kTileBytes;
+    const int kv0 = j * kKvBlock;
+#pragma unroll
+    for (int p = 0; p < kPasses; ++p) {
+      const int seg = (p * 4 + wave) * 1024;
+      const uint8_t* ks = kp + (long long)min(kv0 + k_row[p], kv_last) * a.k_rs + k_col[p];
+      const uint8_t* vs = vp + (long long)min(kv0 + v_row[p], kv_last) * a.v_rs + v_col[p];
+      __builtin_amdgcn_global_load_lds(GLOBAL_PTR(const void, ks), LDS_PTR(void, kb + seg), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds(GLOBAL_PTR(const void, vs), LDS_PTR(void, vb + seg), 16, 0, 0);
+    }
+  };
+
+  // ---- per-lane LDS read offsets ----
+  // K fragment (A operand of S^T): LDS row 32t + qn... the lane's row index inside the 32-row MFMA tile is
+  // lane % 32 and its k-group lane / 32; chunks 4ks+2h and 4ks+2h+1 of that row.
+  int k_off[kKSteps][2];
+#pragma unroll
+  for (int ks = 0; ks < kKSteps; ++ks)
+#pragma unroll
+    for (int e = 0; e < 2; ++e) k_off[ks][e] = tile_offset<D, false>(qn, 4 * ks + 2 * h + e);
+  constexpr int kSubTileStride = 32 * D;  // LDS bytes between S^T sub-tiles (32 rows)
+  // V^T fragment (A operand of O^T = V^T P^T) through ds_read_b64_tr_b8: inside a group of 16 lanes, lanes
+  // 2j and 2j+1 address the two 8-byte halves of kv row j of an 8 x 16 byte block, and lane i receives
+  // byte i of each of the 8 rows: 8 consecutive kv for one head-dim column.
+  const int tr_j = (lane & 15) >> 1, tr_e = lane & 1, tr_g1 = (lane >> 4) & 1;
+  int v_off[kMTiles];
+#pragma unroll
+  for (int mt = 0; mt < kMTiles; ++mt) v_off[mt] = tile_offset<D, true>(32 * h + tr_j, 2 * mt + tr_g1) + 8 * tr_e;
+  constexpr int kTrStride = 8 * D;  // LDS bytes between successive groups of 8 kv rows
+
+  const int n_tiles = CAUSAL ? (min(a.seqlen_k, q0 + kQBlock) + kKvBlock - 1) / kKvBlock
+                             : (a.seqlen_k + kKvBlock - 1) / kKvBlock;
+
+  v16f o_acc[kMTiles];
+#pragma unroll
+  for (int mt = 0; mt < kMTiles; ++mt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) o_acc[mt][i] = 0.f;
+  float m_run = -INFINITY;  // running row max of raw S (both half-lanes of a query hold the same value)
+  float l_run = 0.f;        // this lane's share of the running row sum
+
+  issue_tile(0, 0);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+
+  for (int j = 0; j < n_tiles; ++j) {
+    if (j + 1 < n_tiles) issue_tile(j + 1, (j + 1) & 1);
+    const uint8_t* kb = smem + (j & 1) * kStageBytes;
+    const uint8_t* vb = kb + kTileBytes;
+    const int kv0 = j * kKvBlock;
+    // A wavefront whose 32 query rows all lie before this kv block has nothing to add (causal).
+    const bool active = !CAUSAL || (kv0 <= q_wave0 + kQWave - 1);
+    if (active) {
+      // ---- S^T = K Q^T : two 32(kv) x 32(q) sub-tiles ----
+      v16f s[2];
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[t][i] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < kKSteps; ++ks) {
+          const v4i lo = *LDS_PTR(const v4i, kb + t * kSubTileStride + k_off[ks][0]);
+          const v4i hi = *LDS_PTR(const v4i, kb + t * kSubTileStride + k_off[ks][1]);
+          const v8i kf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+          s[t] = mfma_fp8<E5M2>(kf, qf[ks], s[t]);
+        }
+      }
+      // ---- causal / tail mask: register i of sub-tile t is kv row kv0 + 32h + 16t + i ----
+      const int kv_limit = CAUSAL ? min(q_row, kv_last) : kv_last;  // last kv this query attends to
+      const int wave_limit = CAUSAL ? min(q_wave0, kv_last) : kv_last;
+      const bool need_mask = kv0 + kKvBlock - 1 > wave_limit;
+      if (need_mask) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int i = 0; i < 16; ++i)
+            if (kv0 + 32 * h + 16 * t + i > kv_limit) s[t][i] = -INFINITY;
+      }
+      // ---- online softmax (reference softmax_rescale_o, csrc/flash_attention.cu:233-273) ----
+      float mloc = fmaxf(s[0][0], s[1][0]);
+#pragma unroll
+      for (int i = 1; i < 16; ++i) mloc = fmaxf(mloc, fmaxf(s[0][i], s[1][i]));
+      mloc = lane32_max(mloc);
+      const float m_new = fmaxf(m_run, mloc);
+      if (__any(m_new != m_run)) {
+        const float alpha = (m_run == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((m_run - m_new) * c);
+        l_run *= alpha;
+#pragma unroll
+        for (int mt = 0; mt < kMTiles; ++mt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) o_acc[mt][i] *= alpha;
+        m_run = m_new;
+      }
+      const float mc = (m_new == -INFINITY) ? 0.f : m_new * c;
+      float sum0 = 0.f, sum1 = 0.f;
+      v8i p8;
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[t][i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][i], c, -mc));
+        if (need_mask) {
+          // a masked logit is -inf; force its weight to 0 even when scale <= 0 would give NaN or 1
+#pragma unroll
+          for (int i = 0; i < 16; ++i)
+            if (kv0 + 32 * h + 16 * t + i > kv_limit) s[t][i] = 0.f;
+        }
+#pragma unroll
+        for (int i = 0; i < 16; i += 2) {
+          sum0 += s[t][i];
+          sum1 += s[t][i + 1];
+        }
+#pragma unroll
+        for (int w = 0; w < 4; ++w)
+          p8[4 * t + w] = pack4_fp8<E5M2>(s[t][4 * w], s[t][4 * w + 1], s[t][4 * w + 2], s[t][4 * w + 3]);
+      }
+      l_run += sum0 + sum1;
+      // ---- O^T += V^T P^T ----
+#pragma unroll
+      for (int mt = 0; mt < kMTiles; ++mt) {
+        v8i vf;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const v2i r = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_PTR(v2i, vb + v_off[mt] + g * kTrStride));
+          vf[2 * g] = r[0];
+          vf[2 * g + 1] = r[1];
+        }
+        o_acc[mt] = mfma_fp8<E5M2>(vf, p8, o_acc[mt]);
+      }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+  }
+
+  // ---- epilogue: O / l, convert, store (reference csrc/flash_attention.cu:542-582) ----
+  const float l_tot = lane32_sum(l_run);
+  const float inv = (l_tot == 0.f || l_tot != l_tot) ? 1.f : 1.f / l_tot;
+  if (q_row < a.seqlen_q) {
+    // register i = 4a2 + b2 of tile mt is head-dim column 32mt + 8a2 + 4h + b2
+    if constexpr (OUT == FA8_OUT_FP16) {
+      _Float16* op = (_Float16*)a.o + b * a.o_bs + hd * a.o_hs + (long long)q_row * a.o_rs + 4 * h;
+#pragma unroll
+      for (int mt = 0; mt < kMTiles; ++mt)
+#pragma unroll
+        for (int a2 = 0; a2 < 4; ++a2) {
+          v4h w;
+#pragma unroll
+          for (int b2 = 0; b2 < 4; ++b2) w[b2] = (_Float16)(o_acc[mt][4 * a2 + b2] * inv);
+          *(v4h*)(op + 32 * mt + 8 * a2) = w;
+        }
+    } else {
+      uint8_t* op = (uint8_t*)a.o + b * a.o_bs + hd * a.o_hs + (long long)q_row * a.o_rs + 4 * h;
+#pragma unroll
+      for (int mt = 0; mt < kMTiles; ++mt)
+#pragma unroll
+        for (int a2 = 0; a2 < 4; ++a2) {
+          float x[4];
+#pragma unroll
+          for (int b2 = 0; b2 < 4; ++b2) {
+            const float y = o_acc[mt][4 * a2 + b2] * inv;
+            x[b2] = (y != y) ? y : fminf(fmaxf(y, -448.f), 448.f);  // saturate to finite, keep NaN
+          }
+          *(int*)(op + 32 * mt + 8 * a2) = pack4_fp8<false>(x[0], x[1], x[2], x[3]);
+        }
+    }
+  }
+}
+
+template <int D, bool CAUSAL, bool E5M2, int OUT>
+int launch(const KernelArgs& a, hipStream_t stream) {
+  constexpr int lds_bytes = 2 * 2 * kKvBlock * D;
+  const dim3 grid((unsigned)(a.bh_total * a.n_qblocks));
+  hipLaunchKernelGGL((fa8_fwd_kernel<D, CAUSAL, E5M2, OUT>), grid, dim3(kThreads), lds_bytes, stream, a);
+  return (int)hipGetLastError();
+}
+
+template <int D, bool CAUSAL>
+int launch_types(const Fa8FwdParams* p, const KernelArgs& a, hipStream_t stream) {
+  const bool e5m2 = p->in_dtype == FA8_DTYPE_E5M2;
+  if (p->out_dtype == FA8_OUT_FP16)
+    return e5m2 ? launch<D, CAUSAL, true, FA8_OUT_FP16>(a, stream) : launch<D, CAUSAL, false, FA8_OUT_FP16>(a, stream);
+  // fp8 output: the reference stores O in the input element type; only e4m3 out of e4m3 in is built
+  if (e5m2) return FA8_ERR_UNSUPPORTED;
+  return launch<D, CAUSAL, false, FA8_OUT_E4M3>(a, stream);
+}
+
+bool span_ok(long long outer_stride, long long inner_extent) { return outer_stride >= inner_extent; }
+
+}  // namespace
+
+extern "C" int fa8_fwd_validate(const Fa8FwdParams* p) {
+  if (p == nullptr || p->q == nullptr || p->k == nullptr || p->v == nullptr || p->o == nullptr) return FA8_ERR_NULL;
+  if (p->batch < 1 || p->heads < 1 || p->seqlen_q < 1 || p->seqlen_k < 1 || p->head_dim < 1) return FA8_ERR_SHAPE;
+  if (p->is_causal != 0 && p->is_causal != 1) return FA8_ERR_SHAPE;
+  if (p->is_causal && p->seqlen_q != p->seqlen_k) return FA8_ERR_SHAPE;
+  if ((long long)p->batch * p->heads > 0x7fffffffLL / ((p->seqlen_q + kQBlock - 1) / kQBlock)) return FA8_ERR_SHAPE;
+  if (p->in_dtype != FA8_DTYPE_E4M3 && p->in_dtype != FA8_DTYPE_E5M2) return FA8_ERR_DTYPE;
+  if (p->out_dtype != FA8_OUT_FP16 && p->out_dtype != FA8_OUT_E4M3) return FA8_ERR_DTYPE;
+  if (p->v_layout != FA8_V_ROWS && p->v_layout != FA8_V_TRANSPOSED) return FA8_ERR_DTYPE;
+  if (p->head_dim != 64 && p->head_dim != 128) return FA8_ERR_HEAD_DIM;
+  if (!(p->softmax_scale == p->softmax_scale) || std::isinf(p->softmax_scale)) return FA8_ERR_SCALE;
+  const long long d = p->head_dim;
+  const long long v_rows = p->v_layout == FA8_V_ROWS ? p->seqlen_k : d;
+  const long long v_cols = p->v_layout == FA8_V_ROWS ? d : p->seqlen_k;
+  if (!span_ok(p->q_row_stride, d) || !span_ok(p->q_head_stride, 1) || !span_ok(p->q_batch_stride, 1)) return FA8_ERR_STRIDE;
+  if (!span_ok(p->k_row_stride, d) || !span_ok(p->k_head_stride, 1) || !span_ok(p->k_batch_stride, 1)) return FA8_ERR_STRIDE;
+  if (!span_ok(p->v_row_stride, v_cols) || !span_ok(p->v_head_stride, 1) || !span_ok(p->v_batch_stride, 1)) return FA8_ERR_STRIDE;
+  if (!span_ok(p->o_row_stride, d) || !span_ok(p->o_head_stride, 1) || !span_ok(p->o_batch_stride, 1)) return FA8_ERR_STRIDE;
+  (void)v_rows;
+  // 16-byte vector loads of q/k/v rows, 8-byte (fp16) or 4-byte (fp8) vector stores of o
+  const long long in_strides[] = {p->q_batch_stride, p->q_head_stride, p->q_row_stride, p->k_batch_stride, p->k_head_stride,
+                                  p->k_row_stride,   p->v_batch_stride, p->v_head_stride, p->v_row_stride};
+  for (long long s : in_strides)
+    if (s % 16 != 0) return FA8_ERR_ALIGN;
+  if (((uintptr_t)p->q | (uintptr_t)p->k | (uintptr_t)p->v) % 16 != 0) return FA8_ERR_ALIGN;
+  const long long o_elem = p->out_dtype == FA8_OUT_FP16 ? 2 : 1;
+  const long long o_strides[] = {p->o_batch_stride, p->o_head_stride, p->o_row_stride};
+  for (long long s : o_strides)
+    if ((s * o_elem) % 8 != 0) return FA8_ERR_ALIGN;
+  if ((uintptr_t)p->o % 8 != 0) return FA8_ERR_ALIGN;
+  if (p->v_layout == FA8_V_TRANSPOSED) return FA8_ERR_UNSUPPORTED;
+  if (p->in_dtype == FA8_DTYPE_E5M2 && p->out_dtype == FA8_OUT_E4M3) return FA8_ERR_UNSUPPORTED;
+  return FA8_OK;
+}
+
+extern "C" int fa8_fwd(const Fa8FwdParams* p, void* hip_stream) {
+  const int rc = fa8_fwd_validate(p);
+  if (rc != FA8_OK) return rc;
+  KernelArgs a;
+  a.q = (const uint8_t*)p->q;
+  a.k = (const uint8_t*)p->k;
+  a.v = (const uint8_t*)p->v;
+  a.o = p->o;
+  a.heads = p->heads;
+  a.seqlen_q = p->seqlen_q;
+  a.seqlen_k = p->seqlen_k;
+  a.n_qblocks = (p->seqlen_q + kQBlock - 1) / kQBlock;
+  a.bh_total = p->batch * p->heads;
+  a.scale_log2 = p->softmax_scale * 1.4426950408889634f;
+  a.q_bs = p->q_batch_stride; a.q_hs = p->q_head_stride; a.q_rs = p->q_row_stride;
+  a.k_bs = p->k_batch_stride; a.k_hs = p->k_head_stride; a.k_rs = p->k_row_stride;
+  a.v_bs = p->v_batch_stride; a.v_hs = p->v_head_stride; a.v_rs = p->v_row_stride;
+  a.o_bs = p->o_batch_stride; a.o_hs = p->o_head_stride; a.o_rs = p->o_row_stride;
+  hipStream_t stream = (hipStream_t)hip_stream;
+  if (p->head_dim == 128)
+    return p->is_causal ? launch_types<128, true>(p, a, stream) : launch_types<128, false>(p, a, stream);
+  return p->is_causal ? launch_types<64, true>(p, a, stream) : launch_types<64, false>(p, a, stream);
+}
+
+extern "C" int fa8_query(int what) {
+  switch (what) {
+    case FA8_QUERY_VERSION: return kVersion;
+    case FA8_QUERY_KV_BLOCK: return kKvBlock;
+    case FA8_QUERY_Q_BLOCK: return kQBlock;
+    case FA8_QUERY_KV_ASCENDING: return 1;
+    case FA8_QUERY_THREADS: return kThreads;
+    default: return -1;
+  }
+}
+
+extern "C" const char* fa8_error_string(int code) {
+  switch (code) {
+    case FA8_OK: return "ok";
+    case FA8_ERR_NULL: return "a required pointer is NULL";
+    case FA8_ERR_SHAPE: return "bad shape (a size < 1, too many workgroups, or causal with seqlen_q != seqlen_k)";
+    case FA8_ERR_HEAD_DIM: return "head_dim must be 64 or 128";
+    case FA8_ERR_STRIDE: return "a stride is smaller than the extent it spans";
+    case FA8_ERR_ALIGN: return "q/k/v rows must be 16-byte aligned and o rows 8-byte aligned";
+    case FA8_ERR_DTYPE: return "unknown in_dtype / out_dtype / v_layout code";
+    case FA8_ERR_UNSUPPORTED: return "this build has no kernel for the requested combination";
+    case FA8_ERR_SCALE: return "softmax_scale must be finite";
+    default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown fa8 error code";
+  }
+}

@@ -1,0 +1,418 @@
+/*
+ * fa8_oracle.c -- CPU restatement of the reference FP8 flash-attention forward pipeline.
+ *
+ * TEST INFRASTRUCTURE ONLY.  Nothing under oracle/ is part of the product: only tests/, the smoke
+ * check of __graft_entry__.py and the cpu_baseline leg of bench.py may build, load or call it, and
+ * only as the checker.  The GPU library never links or falls back to this code.
+ *
+ * What it restates (weishengying/cutlass_flash_atten_fp8, all citations into that repository):
+ *   - the KV-block loop of the kernel, csrc/flash_attention.cu:468-534, with its causal loop bound
+ *     (:458) and diagonal mask (mask_within_nblock, :24-71: column > row -> -inf);
+ *   - the online softmax softmax_rescale_o (:233-273) + scale_apply_exp2 (:197-216): row max over the
+ *     RAW logits, alpha = expf((m_prev - m_cur) * scale), P = expf(S * scale - m_cur * scale), the row
+ *     sum taken over the UN-quantised fp32 P (reduce_sum, csrc/utils.h:94-98);
+ *   - convert_float32_to_fp8 (:163-179): P -> fp8 (round-to-nearest-even, saturate to finite) before
+ *     the PV product (:524-533);
+ *   - the epilogue (:542-557): O * (l == 0 || isnan(l) ? 1 : 1/l), then the output conversion
+ *     (fp8 in the reference; fp16 RNE is the primary output of this build).
+ * The block size kBlockN = 64 (:624) is a parameter here because the running max that P is quantised
+ * against depends on it.
+ *
+ * The reference itself cannot be built in this environment (CUDA inline PTX, un-vendored CUTLASS), so
+ * there is no oracle/_ref.  What pins this file instead (tests/test_e4m3_codec.py, tests/test_oracle_*.py):
+ *   - fp8 codecs: exhaustive decode against the closed form, encode on every midpoint between adjacent
+ *     codes, cross-checked against torch's CPU cast;
+ *   - fa8o_fwd_rows: an independent numpy restatement, closed-form known answers (dominant logit, equal
+ *     keys, scale = 0, causal row 0, constant V), brute-force fp64 triple loops on tiny inputs, and
+ *     equality with fp64 softmax attention when P quantisation is switched off.
+ * Not pinned (hardware details no CPU reproduces, both far below the tolerance): the accumulation order
+ * inside the sm_89 tensor core and the ulp behaviour of __expf under --use_fast_math.
+ */
+#include <math.h>
+#include <stddef.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#define FA8O_E4M3 0
+#define FA8O_E5M2 1
+#define FA8O_OUT_FP16 0
+#define FA8O_OUT_E4M3 1
+#define FA8O_OUT_F32 2 /* un-rounded fp32 result, for tests */
+
+/* ---------------- fp8 / fp16 codecs (closed forms, no tables) ---------------- */
+
+/* OCP e4m3fn: 1-4-3, bias 7, no infinities, NaN = S.1111.111, max 448, min subnormal 2^-9. */
+float fa8o_e4m3_to_f32(uint8_t c) {
+  const int s = c >> 7, e = (c >> 3) & 15, m = c & 7;
+  float v;
+  if (e == 15 && m == 7) return NAN;
+  if (e == 0)
+    v = ldexpf((float)m, -9);
+  else
+    v = ldexpf((float)(8 + m), e - 10);
+  return s ? -v : v;
+}
+
+/* OCP e5m2: 1-5-2, bias 15, IEEE-like infinities and NaNs, max 57344, min subnormal 2^-16. */
+float fa8o_e5m2_to_f32(uint8_t c) {
+  const int s = c >> 7, e = (c >> 2) & 31, m = c & 3;
+  float v;
+  if (e == 31) return m ? NAN : (s ? -INFINITY : INFINITY);
+  if (e == 0)
+    v = ldexpf((float)m, -16);
+  else
+    v = ldexpf((float)(4 + m), e - 17);
+  return s ? -v : v;
+}
+
+/* Round |x| to a grid with `mbits` mantissa bits and minimum exponent `emin` (ties to even). */
+static float round_to_grid(float ax, int mbits, int emin) {
+  int e;
+  (void)frexpf(ax, &e); /* ax = f * 2^e, f in [0.5, 1) */
+  int E = e - 1;
+  if (E < emin) E = emin;
+  const float q = ldexpf(1.0f, E - mbits);
+  return nearbyintf(ax / q) * q; /* division by a power of two is exact; default mode = ties to even */
+}
+
+/* fp32 -> e4m3fn, round to nearest even, saturate to +-448 (what __nv_fp8x2_e4m3 does, reference :166-176). */
+uint8_t fa8o_f32_to_e4m3(float x) {
+  const uint8_t s = signbit(x) ? 0x80 : 0;
+  float ax = fabsf(x);
+  if (ax != ax) return s | 0x7F;
+  if (ax > 448.0f) ax = 448.0f;
+  if (ax == 0.0f) return s;
+  const float v = round_to_grid(ax, 3, -6);
+  if (v == 0.0f) return s;
+  if (v < 0.015625f) return s | (uint8_t)(v * 512.0f); /* subnormal: m * 2^-9 */
+  int e;
+  const float f = frexpf(v, &e); /* v = f * 2^e */
+  const int E = e - 1;
+  const int m = (int)((f * 2.0f - 1.0f) * 8.0f);
+  return s | (uint8_t)(((E + 7) << 3) | m);
+}
+
+/* fp32 -> e5m2, round to nearest even, saturate to +-57344. */
+uint8_t fa8o_f32_to_e5m2(float x) {
+  const uint8_t s = signbit(x) ? 0x80 : 0;
+  float ax = fabsf(x);
+  if (ax != ax) return s | 0x7F;
+  if (ax > 57344.0f) ax = 57344.0f;
+  if (ax == 0.0f) return s;
+  const float v = round_to_grid(ax, 2, -14);
+  if (v == 0.0f) return s;
+  if (v < 6.103515625e-05f) return s | (uint8_t)(v * 65536.0f); /* subnormal: m * 2^-16 */
+  int e;
+  const float f = frexpf(v, &e);
+  const int E = e - 1;
+  const int m = (int)((f * 2.0f - 1.0f) * 4.0f);
+  return s | (uint8_t)(((E + 15) << 2) | m);
+}
+
+/* fp32 -> IEEE binary16, round to nearest even, overflow to infinity. */
+uint16_t fa8o_f32_to_f16(float x) {
+  const uint16_t s = signbit(x) ? 0x8000 : 0;
+  float ax = fabsf(x);
+  if (ax != ax) return s | 0x7E00;
+  if (isinf(ax)) return s | 0x7C00;
+  if (ax == 0.0f) return s;
+  if (ax >= 65520.0f) return s | 0x7C00; /* rounds up past the largest half */
+  const float v = round_to_grid(ax, 10, -14);
+  if (v == 0.0f) return s;
+  if (v < 6.103515625e-05f) return s | (uint16_t)(v * 16777216.0f); /* subnormal: m * 2^-24 */
+  int e;
+  const float f = frexpf(v, &e);
+  const int E = e - 1;
+  const int m = (int)((f * 2.0f - 1.0f) * 1024.0f);
+  return s | (uint16_t)(((E + 15) << 10) | m);
+}
+
+float fa8o_f16_to_f32(uint16_t c) {
+  const int s = c >> 15, e = (c >> 10) & 31, m = c & 1023;
+  float v;
+  if (e == 31) return m ? NAN : (s ? -INFINITY : INFINITY);
+  if (e == 0)
+    v = ldexpf((float)m, -24);
+  else
+    v = ldexpf((float)(1024 + m), e - 25);
+  return s ? -v : v;
+}
+
+/* ---------------- the pipeline ---------------- */
+
+typedef struct Fa8OracleArgs {
+  const uint8_t* q; /* [B,H,Nq,d] contiguous */
+  const uint8_t* k; /* [B,H,Nk,d] contiguous */
+  const uint8_t* v; /* [B,H,Nk,d] contiguous, or [B,H,d,Nk] when v_transposed */
+  void* o;          /* [B,H,Nq,d]: uint16 (fp16 bits), uint8 (e4m3) or float */
+  int32_t batch, heads, seqlen_q, seqlen_k, head_dim;
+  int32_t is_causal;
+  int32_t kv_block;    /* columns per online-softmax step; the reference uses 64 */
+  int32_t in_dtype;    /* FA8O_E4M3 / FA8O_E5M2 */
+  int32_t out_dtype;   /* FA8O_OUT_* */
+  int32_t v_transposed;
+  int32_t quantize_p;  /* 1 = reference behaviour; 0 = keep P in fp32 (textbook flash attention) */
+  int32_t exp2_form;   /* 0 = expf(s*scale - m*scale) as the reference; 1 = exp2f(fma(s, c, -m*c)), c = scale*log2(e) */
+  float softmax_scale;
+  /* Optional rounding-flip allowance, see oracle_row.  flip_allow is float [B,H,n_rows] or NULL. */
+  float* flip_allow;
+  float logit_rel_err; /* bound on |S_device - S_exact| / sum_k |q_k k_k| of the matrix core being checked */
+} Fa8OracleArgs;
+
+/* 256-entry decode tables filled from the closed forms above (idempotent, so concurrent first calls are harmless). */
+static float g_lut[2][256];
+static volatile int g_lut_ready = 0;
+static void init_lut(void) {
+  if (g_lut_ready) return;
+  for (int c = 0; c < 256; ++c) {
+    g_lut[FA8O_E4M3][c] = fa8o_e4m3_to_f32((uint8_t)c);
+    g_lut[FA8O_E5M2][c] = fa8o_e5m2_to_f32((uint8_t)c);
+  }
+  g_lut_ready = 1;
+}
+
+/* fp32 dot product with 8 interleaved partial sums combined as a tree.  The accumulation order of the tensor
+ * core is unspecified (and fp8 x fp8 products are exact in fp32), so any fixed fp32 order is as faithful as another. */
+static float dot_f32(const float* x, const float* y, int d) {
+  float s[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  int i = 0;
+  for (; i + 8 <= d; i += 8)
+    for (int u = 0; u < 8; ++u) s[u] += x[i + u] * y[i + u];
+  for (; i < d; ++i) s[i & 7] += x[i] * y[i];
+  return ((s[0] + s[1]) + (s[2] + s[3])) + ((s[4] + s[5]) + (s[6] + s[7]));
+}
+
+static float dot_abs_f32(const float* x, const float* y, int d) {
+  float s = 0.0f;
+  for (int i = 0; i < d; ++i) s += fabsf(x[i] * y[i]);
+  return s;
+}
+
+/* Relative distance of p (0 < p <= max) to the nearest point where its fp8 rounding changes, and the size of
+ * that change (*quantum).  Grid: mbits mantissa bits, minimum exponent emin. */
+static float tie_distance(float p, int mbits, int emin, float* quantum) {
+  int e;
+  (void)frexpf(p, &e);
+  int E = e - 1;
+  if (E < emin) E = emin;
+  const float u = ldexpf(1.0f, E - mbits);
+  const float t = p / u;                 /* exact */
+  const float frac = t - floorf(t);      /* position between two grid points */
+  *quantum = u;
+  return fabsf(frac - 0.5f) * u / p;
+}
+
+/* One query row.  kf/vf are the dequantised K [Nk,d] and V [Nk,d] of this head; p is scratch [kv_block]. */
+static void oracle_row(const Fa8OracleArgs* a, const float* qrow, const float* kf, const float* vf, int i, float* p,
+                       float* acc /* [d] */, float* flip_allow) {
+  /* flip_allow (optional): P is rounded to 3 (e4m3) or 2 (e5m2) mantissa bits, so a device whose logits differ
+   * from the exact ones by a few 1e-5 of sum|q_k k_k| (matrix cores do not accumulate in IEEE fp32) can round a
+   * P that lies next to a rounding boundary the other way: a legitimate one-quantum difference that changes
+   * O[i,:] by quantum * V[j,:] / l.  *flip_allow returns the sum of those possible changes (times max|V[j,:]|)
+   * over the columns whose P is within reach of a boundary given a->logit_rel_err. */
+  const int d = a->head_dim, nk = a->seqlen_k, bc = a->kv_block;
+  float allow = 0.0f;
+  const int mbits = a->in_dtype == FA8O_E5M2 ? 2 : 3, emin = a->in_dtype == FA8O_E5M2 ? -14 : -6;
+  const float scale = a->softmax_scale;
+  const float c2 = scale * 1.4426950408889634f;
+  float m = -INFINITY, l = 0.0f;
+  for (int x = 0; x < d; ++x) acc[x] = 0.0f;
+  /* Reference loop bound (:458): every block that starts before the end of the row's q block.  Blocks that
+   * start after column i are fully masked for this row (m, l and O unchanged), so the loop may stop at j0 <= i. */
+  const int j_end = a->is_causal ? (i + 1 < nk ? i + 1 : nk) : nk; /* columns [0, j_end) are visible */
+  for (int j0 = 0; j0 < j_end; j0 += bc) {
+    const int jn = j0 + bc < nk ? j0 + bc : nk; /* the block covers columns [j0, jn) */
+    float bmax = -INFINITY;
+    for (int j = j0; j < jn; ++j) {
+      /* S = q . k_j in fp32 (:487); causal mask: column > row -> -inf (:62-64) */
+      const float s = j < j_end ? dot_f32(qrow, kf + (size_t)j * d, d) : -INFINITY;
+      p[j - j0] = s;
+      if (s > bmax) bmax = s;
+    }
+    const float m_new = m > bmax ? m : bmax; /* max over the raw logits (:238, :249) */
+    if (m != -INFINITY) {                    /* not the first block: rescale l and O (:258-261) */
+      const float alpha = a->exp2_form ? exp2f((m - m_new) * c2) : expf((m - m_new) * scale);
+      l *= alpha;
+      allow *= alpha;
+      for (int x = 0; x < d; ++x) acc[x] *= alpha;
+    }
+    const float m_scaled = (m_new == -INFINITY) ? 0.0f : (a->exp2_form ? m_new * c2 : m_new * scale); /* :207 */
+    float rowsum = 0.0f;
+    for (int j = j0; j < jn; ++j) {
+      float pj = 0.0f; /* masked columns weigh 0 (expf(-inf) in the reference) */
+      if (j < j_end) pj = a->exp2_form ? exp2f(fmaf(p[j - j0], c2, -m_scaled)) : expf(p[j - j0] * scale - m_scaled);
+      rowsum += pj; /* the denominator uses the fp32 P (:240, :268-271) */
+      if (flip_allow && a->quantize_p && j < j_end && pj > 0.0f) {
+        float quantum;
+        const float dist = tie_distance(pj, mbits, emin, &quantum);
+        /* the device logit and the device row max may each be off by logit_rel_err * sum|terms| */
+        const float reach = 2.0f * fabsf(scale) * a->logit_rel_err * dot_abs_f32(qrow, kf + (size_t)j * d, d);
+        if (dist <= reach) {
+          float vmax = 0.0f;
+          for (int x = 0; x < d; ++x) vmax = fmaxf(vmax, fabsf(vf[(size_t)j * d + x]));
+          allow += quantum * vmax;
+        }
+      }
+      if (a->quantize_p) /* P -> fp8 before PV (:524) */
+        pj = a->in_dtype == FA8O_E5M2 ? g_lut[FA8O_E5M2][fa8o_f32_to_e5m2(pj)] : g_lut[FA8O_E4M3][fa8o_f32_to_e4m3(pj)];
+      p[j - j0] = pj;
+    }
+    l += rowsum;
+    for (int j = j0; j < jn; ++j) { /* O += P8 V (:533), fp32 accumulation */
+      const float pj = p[j - j0];
+      if (pj == 0.0f) continue;
+      const float* vr = vf + (size_t)j * d;
+      for (int x = 0; x < d; ++x) acc[x] += pj * vr[x];
+    }
+    m = m_new;
+  }
+  const float inv = (l == 0.0f || l != l) ? 1.0f : 1.0f / l; /* :545-553 */
+  for (int x = 0; x < d; ++x) acc[x] *= inv;
+  if (flip_allow) *flip_allow = allow * inv;
+}
+
+static void dequant_head(const Fa8OracleArgs* a, int bh, float* kf, float* vf) {
+  const int nk = a->seqlen_k, d = a->head_dim;
+  const float* lut = g_lut[a->in_dtype == FA8O_E5M2 ? FA8O_E5M2 : FA8O_E4M3];
+  const uint8_t* kq = a->k + (size_t)bh * nk * d;
+  const uint8_t* vq = a->v + (size_t)bh * nk * d;
+  if (kf)
+    for (size_t t = 0; t < (size_t)nk * d; ++t) kf[t] = lut[kq[t]];
+  for (int j = 0; j < nk; ++j)
+    for (int x = 0; x < d; ++x) vf[(size_t)j * d + x] = lut[a->v_transposed ? vq[(size_t)x * nk + j] : vq[(size_t)j * d + x]];
+}
+
+/*
+ * The forward pass for the query rows rows[0..n_rows) of every (batch, head) (rows == NULL: all rows, n_rows
+ * ignored).  o is [B,H,n_rows,d] in the element type out_dtype selects.  Row subsets let the parity tests check
+ * the largest configurations on a sample of rows in seconds.
+ */
+int fa8o_fwd_rows(const Fa8OracleArgs* a, const int32_t* rows, int32_t n_rows) {
+  const int B = a->batch, H = a->heads, nq = a->seqlen_q, nk = a->seqlen_k, d = a->head_dim;
+  if (B < 1 || H < 1 || nq < 1 || nk < 1 || d < 1 || a->kv_block < 1) return -1;
+  const int nr = rows ? n_rows : nq;
+  if (nr < 1) return -1;
+  if (rows)
+    for (int r = 0; r < nr; ++r)
+      if (rows[r] < 0 || rows[r] >= nq) return -1;
+  init_lut();
+  const float* lut = g_lut[a->in_dtype == FA8O_E5M2 ? FA8O_E5M2 : FA8O_E4M3];
+  int failed = 0;
+#ifdef _OPENMP
+#pragma omp parallel
+#endif
+  {
+    float* kf = (float*)malloc((size_t)nk * d * sizeof(float));
+    float* vf = (float*)malloc((size_t)nk * d * sizeof(float));
+    float* qrow = (float*)malloc((size_t)d * sizeof(float));
+    float* acc = (float*)malloc((size_t)d * sizeof(float));
+    float* p = (float*)malloc((size_t)a->kv_block * sizeof(float));
+    if (!kf || !vf || !qrow || !acc || !p) {
+#ifdef _OPENMP
+#pragma omp atomic write
+#endif
+      failed = 1;
+    }
+    /* every thread walks the heads in order and takes a share of each head's rows */
+    for (int bh = 0; bh < B * H; ++bh) {
+      if (!failed) dequant_head(a, bh, kf, vf);
+#ifdef _OPENMP
+#pragma omp for schedule(dynamic, 8) nowait
+#endif
+      for (int r = 0; r < nr; ++r) {
+        if (failed) continue;
+        const int i = rows ? rows[r] : r;
+        const uint8_t* qq = a->q + ((size_t)bh * nq + i) * d;
+        for (int x = 0; x < d; ++x) qrow[x] = lut[qq[x]];
+        oracle_row(a, qrow, kf, vf, i, p, acc, a->flip_allow ? a->flip_allow + (size_t)bh * nr + r : NULL);
+        const size_t o0 = ((size_t)bh * nr + r) * d;
+        if (a->out_dtype == FA8O_OUT_FP16) {
+          uint16_t* o = (uint16_t*)a->o;
+          for (int x = 0; x < d; ++x) o[o0 + x] = fa8o_f32_to_f16(acc[x]);
+        } else if (a->out_dtype == FA8O_OUT_E4M3) {
+          uint8_t* o = (uint8_t*)a->o;
+          for (int x = 0; x < d; ++x) o[o0 + x] = fa8o_f32_to_e4m3(acc[x]);
+        } else {
+          float* o = (float*)a->o;
+          for (int x = 0; x < d; ++x) o[o0 + x] = acc[x];
+        }
+      }
+    }
+    free(kf); free(vf); free(qrow); free(acc); free(p);
+  }
+  return failed ? -2 : 0;
+}
+
+/* Exact softmax attention in fp64 on the dequantised inputs (no P quantisation, no blocks): the textbook result
+ * the fp8 pipeline approximates.  o is double [B,H,n_rows,d]; rows == NULL means all rows. */
+int fa8o_attention_f64(const Fa8OracleArgs* a, const int32_t* rows, int32_t n_rows, double* o) {
+  const int B = a->batch, H = a->heads, nq = a->seqlen_q, nk = a->seqlen_k, d = a->head_dim;
+  if (B < 1 || H < 1 || nq < 1 || nk < 1 || d < 1) return -1;
+  const int nr = rows ? n_rows : nq;
+  if (nr < 1) return -1;
+  if (rows)
+    for (int r = 0; r < nr; ++r)
+      if (rows[r] < 0 || rows[r] >= nq) return -1;
+  init_lut();
+  const float* lut = g_lut[a->in_dtype == FA8O_E5M2 ? FA8O_E5M2 : FA8O_E4M3];
+  int failed = 0;
+#ifdef _OPENMP
+#pragma omp parallel
+#endif
+  {
+    double* s = (double*)malloc((size_t)nk * sizeof(double));
+    float* kf = (float*)malloc((size_t)nk * d * sizeof(float));
+    float* vf = (float*)malloc((size_t)nk * d * sizeof(float));
+    if (!s || !kf || !vf) {
+#ifdef _OPENMP
+#pragma omp atomic write
+#endif
+      failed = 1;
+    }
+    for (int bh = 0; bh < B * H; ++bh) {
+      if (!failed) dequant_head(a, bh, kf, vf);
+#ifdef _OPENMP
+#pragma omp for schedule(dynamic, 8) nowait
+#endif
+      for (int r = 0; r < nr; ++r) {
+        if (failed) continue;
+        const int i = rows ? rows[r] : r;
+        const uint8_t* qq = a->q + ((size_t)bh * nq + i) * d;
+        const int j_end = a->is_causal ? (i + 1 < nk ? i + 1 : nk) : nk;
+        double mx = -INFINITY;
+        for (int j = 0; j < j_end; ++j) {
+          double acc = 0.0;
+          for (int x = 0; x < d; ++x) acc += (double)lut[qq[x]] * (double)kf[(size_t)j * d + x];
+          s[j] = acc * (double)a->softmax_scale;
+          if (s[j] > mx) mx = s[j];
+        }
+        double den = 0.0;
+        for (int j = 0; j < j_end; ++j) {
+          s[j] = exp(s[j] - mx);
+          den += s[j];
+        }
+        double* orow = o + ((size_t)bh * nr + r) * d;
+        for (int x = 0; x < d; ++x) orow[x] = 0.0;
+        for (int j = 0; j < j_end; ++j) {
+          const double w = s[j] / den;
+          for (int x = 0; x < d; ++x) orow[x] += w * (double)vf[(size_t)j * d + x];
+        }
+      }
+    }
+    free(s); free(kf); free(vf);
+  }
+  return failed ? -2 : 0;
+}
+
+int fa8o_num_threads(void) {
+#ifdef _OPENMP
+  return omp_get_max_threads();
+#else
+  return 1;
+#endif
+}

@@ -1,0 +1,123 @@
+"""ctypes front end of oracle/fa8_oracle.c (the C restatement of the reference pipeline).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by the smoke check and by bench.py's cpu_baseline leg.
+The arrays are numpy uint8 views of the fp8 tensors, so the oracle never depends on torch's fp8 casts.
+Reference lines each step follows are cited in fa8_oracle.c.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "liboracle.so")
+
+E4M3, E5M2 = 0, 1
+OUT_FP16, OUT_E4M3, OUT_F32 = 0, 1, 2
+
+
+class _Args(ctypes.Structure):
+    _fields_ = [
+        ("q", ctypes.c_void_p), ("k", ctypes.c_void_p), ("v", ctypes.c_void_p), ("o", ctypes.c_void_p),
+        ("batch", ctypes.c_int32), ("heads", ctypes.c_int32), ("seqlen_q", ctypes.c_int32),
+        ("seqlen_k", ctypes.c_int32), ("head_dim", ctypes.c_int32), ("is_causal", ctypes.c_int32),
+        ("kv_block", ctypes.c_int32), ("in_dtype", ctypes.c_int32), ("out_dtype", ctypes.c_int32),
+        ("v_transposed", ctypes.c_int32), ("quantize_p", ctypes.c_int32), ("exp2_form", ctypes.c_int32),
+        ("softmax_scale", ctypes.c_float), ("flip_allow", ctypes.c_void_p), ("logit_rel_err", ctypes.c_float),
+    ]
+
+
+def build(force=False):
+    """Compile liboracle.so with the Makefile next to this file (gcc, a second or two)."""
+    if force or not os.path.exists(_LIB_PATH) or os.path.getmtime(_LIB_PATH) < os.path.getmtime(
+            os.path.join(_HERE, "fa8_oracle.c")):
+        subprocess.run(["make", "-C", _HERE, "-B", "liboracle.so"], check=True, capture_output=True)
+    return _LIB_PATH
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        build()
+        L = ctypes.CDLL(_LIB_PATH)
+        L.fa8o_e4m3_to_f32.restype = ctypes.c_float
+        L.fa8o_e4m3_to_f32.argtypes = [ctypes.c_uint8]
+        L.fa8o_e5m2_to_f32.restype = ctypes.c_float
+        L.fa8o_e5m2_to_f32.argtypes = [ctypes.c_uint8]
+        L.fa8o_f32_to_e4m3.restype = ctypes.c_uint8
+        L.fa8o_f32_to_e4m3.argtypes = [ctypes.c_float]
+        L.fa8o_f32_to_e5m2.restype = ctypes.c_uint8
+        L.fa8o_f32_to_e5m2.argtypes = [ctypes.c_float]
+        L.fa8o_f32_to_f16.restype = ctypes.c_uint16
+        L.fa8o_f32_to_f16.argtypes = [ctypes.c_float]
+        L.fa8o_f16_to_f32.restype = ctypes.c_float
+        L.fa8o_f16_to_f32.argtypes = [ctypes.c_uint16]
+        L.fa8o_fwd_rows.restype = ctypes.c_int
+        L.fa8o_fwd_rows.argtypes = [ctypes.POINTER(_Args), ctypes.c_void_p, ctypes.c_int32]
+        L.fa8o_attention_f64.restype = ctypes.c_int
+        L.fa8o_attention_f64.argtypes = [ctypes.POINTER(_Args), ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p]
+        L.fa8o_num_threads.restype = ctypes.c_int
+        _lib = L
+    return _lib
+
+
+def _prep(q, k, v, v_transposed):
+    q = np.ascontiguousarray(q, dtype=np.uint8)
+    k = np.ascontiguousarray(k, dtype=np.uint8)
+    v = np.ascontiguousarray(v, dtype=np.uint8)
+    assert q.ndim == 4 and k.ndim == 4 and v.ndim == 4
+    B, H, nq, d = q.shape
+    nk = k.shape[2]
+    assert k.shape == (B, H, nk, d)
+    assert v.shape == ((B, H, d, nk) if v_transposed else (B, H, nk, d))
+    return q, k, v, B, H, nq, nk, d
+
+
+def forward(q, k, v, scale, causal=False, kv_block=64, rows=None, in_dtype=E4M3, out_dtype=OUT_FP16,
+            v_transposed=False, quantize_p=True, exp2_form=False, logit_rel_err=None):
+    """The reference pipeline on uint8 views of fp8 q/k/v [B,H,N,d].
+
+    Returns [B,H,n_rows,d] as float16 (OUT_FP16), uint8 e4m3 codes (OUT_E4M3) or float32 (OUT_F32).
+    rows: optional 1-D int array of query rows to evaluate for every (batch, head).
+    logit_rel_err: when given, also returns flip_allow float32 [B,H,n_rows]: how much O[row,:] may legitimately
+    move because some P sits within reach of an fp8 rounding boundary for a device whose logits are accurate
+    to logit_rel_err * sum_k|q_k k_k| (see oracle_row in fa8_oracle.c).
+    """
+    q, k, v, B, H, nq, nk, d = _prep(q, k, v, v_transposed)
+    rows_arr = None if rows is None else np.ascontiguousarray(rows, dtype=np.int32)
+    nr = nq if rows_arr is None else int(rows_arr.shape[0])
+    np_dtype = {OUT_FP16: np.uint16, OUT_E4M3: np.uint8, OUT_F32: np.float32}[out_dtype]
+    o = np.zeros((B, H, nr, d), dtype=np_dtype)
+    allow = None if logit_rel_err is None else np.zeros((B, H, nr), dtype=np.float32)
+    a = _Args(q.ctypes.data, k.ctypes.data, v.ctypes.data, o.ctypes.data, B, H, nq, nk, d, int(bool(causal)),
+              int(kv_block), int(in_dtype), int(out_dtype), int(bool(v_transposed)), int(bool(quantize_p)),
+              int(bool(exp2_form)), float(scale), None if allow is None else allow.ctypes.data,
+              0.0 if logit_rel_err is None else float(logit_rel_err))
+    rc = lib().fa8o_fwd_rows(ctypes.byref(a), None if rows_arr is None else rows_arr.ctypes.data, nr)
+    if rc != 0:
+        raise RuntimeError(f"fa8o_fwd_rows failed with {rc}")
+    res = o.view(np.float16) if out_dtype == OUT_FP16 else o
+    return res if allow is None else (res, allow)
+
+
+def attention_f64(q, k, v, scale, causal=False, rows=None, in_dtype=E4M3, v_transposed=False):
+    """Exact fp64 softmax attention on the dequantised inputs; float64 [B,H,n_rows,d]."""
+    q, k, v, B, H, nq, nk, d = _prep(q, k, v, v_transposed)
+    rows_arr = None if rows is None else np.ascontiguousarray(rows, dtype=np.int32)
+    nr = nq if rows_arr is None else int(rows_arr.shape[0])
+    o = np.zeros((B, H, nr, d), dtype=np.float64)
+    a = _Args(q.ctypes.data, k.ctypes.data, v.ctypes.data, None, B, H, nq, nk, d, int(bool(causal)), 64,
+              int(in_dtype), OUT_F32, int(bool(v_transposed)), 0, 0, float(scale), None, 0.0)
+    rc = lib().fa8o_attention_f64(ctypes.byref(a), None if rows_arr is None else rows_arr.ctypes.data, nr,
+                                  o.ctypes.data)
+    if rc != 0:
+        raise RuntimeError(f"fa8o_attention_f64 failed with {rc}")
+    return o
+
+
+def num_threads():
+    return int(lib().fa8o_num_threads())

@@ -1,0 +1,90 @@
+"""Second, independent restatement of the reference pipeline in numpy (vectorised over query rows).
+
+TEST INFRASTRUCTURE ONLY.  It shares no code with fa8_oracle.c: the fp8 codec here is table based
+(decode by the closed form into a sorted table, encode by nearest-value search with ties to the even
+code), and the block loop works on whole [Nq, Bc] score panels.  tests/ use it to pin the C oracle.
+Follows reference csrc/flash_attention.cu:468-557 (loop), :197-273 (online softmax), :163-179 (P -> fp8).
+"""
+import numpy as np
+
+
+def _decode_table(ebits, mbits, bias, fn):
+    """All 256 codes -> float64 by the closed form; fn=True: e4m3fn (no inf, single NaN mantissa)."""
+    out = np.zeros(256, dtype=np.float64)
+    emax = (1 << ebits) - 1
+    for c in range(256):
+        s = -1.0 if c & 0x80 else 1.0
+        e = (c >> mbits) & emax
+        m = c & ((1 << mbits) - 1)
+        if fn and e == emax and m == (1 << mbits) - 1:
+            out[c] = np.nan
+        elif (not fn) and e == emax:
+            out[c] = np.nan if m else s * np.inf
+        elif e == 0:
+            out[c] = s * m * 2.0 ** (1 - bias - mbits)
+        else:
+            out[c] = s * (1 + m / (1 << mbits)) * 2.0 ** (e - bias)
+    return out
+
+
+E4M3_TABLE = _decode_table(4, 3, 7, True)
+E5M2_TABLE = _decode_table(5, 2, 15, False)
+
+
+def decode(codes, fmt="e4m3"):
+    table = E4M3_TABLE if fmt == "e4m3" else E5M2_TABLE
+    return table[np.asarray(codes, dtype=np.uint8)]
+
+
+def encode_rne_sat(x, fmt="e4m3"):
+    """float -> fp8 code, nearest value, ties to the even code, saturating to the largest finite value."""
+    table = E4M3_TABLE if fmt == "e4m3" else E5M2_TABLE
+    x = np.asarray(x, dtype=np.float64)
+    pos_codes = np.array([c for c in range(128) if np.isfinite(table[c])], dtype=np.int64)
+    pos_vals = table[pos_codes]  # ascending: code order equals value order for positive fp8
+    ax = np.minimum(np.abs(x), pos_vals[-1])
+    hi = np.clip(np.searchsorted(pos_vals, ax, side="left"), 0, len(pos_vals) - 1)
+    lo = np.clip(hi - 1, 0, len(pos_vals) - 1)
+    d_hi = np.abs(pos_vals[hi] - ax)
+    d_lo = np.abs(ax - pos_vals[lo])
+    pick_lo = (d_lo < d_hi) | ((d_lo == d_hi) & (pos_codes[lo] % 2 == 0))
+    code = np.where(pick_lo, pos_codes[lo], pos_codes[hi]).astype(np.uint8)
+    code = np.where(np.signbit(x), code | 0x80, code).astype(np.uint8)
+    return np.where(np.isnan(x), np.uint8(0x7F), code).astype(np.uint8)
+
+
+def forward(q, k, v, scale, causal=False, kv_block=64, fmt="e4m3", quantize_p=True, out="fp16"):
+    """q, k, v: uint8 [B,H,N,d] fp8 codes.  Returns float16 (out='fp16') or float32 (out='f32')."""
+    q = np.asarray(q, dtype=np.uint8)
+    B, H, nq, d = q.shape
+    nk = k.shape[2]
+    qf = decode(q, fmt).astype(np.float32)
+    kf = decode(k, fmt).astype(np.float32)
+    vf = decode(v, fmt).astype(np.float32)
+    scale = np.float32(scale)
+    res = np.zeros((B, H, nq, d), dtype=np.float32)
+    rows = np.arange(nq)[:, None]
+    for b in range(B):
+        for h in range(H):
+            m = np.full(nq, -np.inf, dtype=np.float32)
+            l = np.zeros(nq, dtype=np.float32)
+            o = np.zeros((nq, d), dtype=np.float32)
+            for j0 in range(0, nk, kv_block):
+                cols = np.arange(j0, min(j0 + kv_block, nk))[None, :]
+                s = (qf[b, h] @ kf[b, h, j0:j0 + kv_block].T).astype(np.float32)
+                visible = (cols <= rows) if causal else np.ones_like(s, dtype=bool)
+                s = np.where(visible, s, np.float32(-np.inf))
+                m_new = np.maximum(m, s.max(axis=1))
+                with np.errstate(invalid="ignore"):
+                    alpha = np.where(np.isneginf(m), np.float32(0), np.exp((m - m_new) * scale)).astype(np.float32)
+                m_scaled = np.where(np.isneginf(m_new), np.float32(0), m_new * scale).astype(np.float32)
+                with np.errstate(invalid="ignore"):
+                    p = np.exp(s * scale - m_scaled[:, None]).astype(np.float32)
+                p = np.where(visible, p, np.float32(0))
+                l = l * alpha + p.sum(axis=1, dtype=np.float32)
+                p8 = decode(encode_rne_sat(p, fmt), fmt).astype(np.float32) if quantize_p else p
+                o = o * alpha[:, None] + (p8 @ vf[b, h, j0:j0 + kv_block]).astype(np.float32)
+                m = m_new
+            inv = np.where((l == 0) | np.isnan(l), np.float32(1), np.float32(1) / l).astype(np.float32)
+            res[b, h] = o * inv[:, None]
+    return res.astype(np.float16) if out == "fp16" else res
