@@ -1,0 +1,148 @@
+#!/usr/bin/env python3
+"""Benchmark of the FP8 flash-attention forward hot path on one MI355X.
+
+A step is one call of `attention_cutlass_fp8.flash_attention_v2_cutlass(q, k, v, is_causal, softmax_scale)` on the
+headline workload (B=2, H=32, N=4096, d=128, non-causal, e4m3 inputs drawn N(0,1), fp16 output) with q/k/v already
+resident in HBM.  Prints ONE JSON line: TFLOP/s = 4*B*H*N^2*d / t (halved for causal workloads), the fraction of the
+MI355X dense FP8 MFMA peak, and a CPU baseline (the reference's naive attention restated in PyTorch, timed on the host
+cores of the same machine on a bounded sample of heads).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3] [--no-cpu-baseline]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+FP8_MFMA_PEAK_TFLOPS = 5000.0  # MI355X dense FP8 matrix peak (5.0 PFLOP/s)
+HBM_PEAK_GBPS = 8000.0
+
+# HBM bytes per launch of the headline workload read by rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), each scaled by
+# what the same counter reads for a plain copy kernel of known size; see profiles/.  None until measured.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="cfg3", help="cfg1..cfg5 (cfg3 is the headline)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the baseline sample")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (the path shards over batch*heads with no communication; "
+              "see DESIGN.md); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import cutlass_flash_atten_fp8_amd as fa
+    from cutlass_flash_atten_fp8_amd import inputs
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(3)
+    ext = fa.load_extension()  # raises if the native code has not been built: there is no fallback path
+    cfg = inputs.CONFIGS[args.workload]
+    scale = inputs.softmax_scale(cfg)
+    causal = cfg["causal"]
+    dev = torch.device("cuda:0")
+    q8, k8, v8 = inputs.make_qkv(cfg)
+    q, k, v = q8.to(dev), k8.to(dev), v8.to(dev)
+    flops = inputs.flops(cfg)
+
+    def step():
+        return ext.flash_attention_v2_cutlass(q, k, v, causal, scale)[0]
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    # whole-step wall clock: exactly `steps` steps between two device synchronisations
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # kernel duration: HIP events on the stream the kernel is launched on (torch's current stream), one pair per launch
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    for e0, e1 in evs:
+        e0.record()
+        step()
+        e1.record()
+    torch.cuda.synchronize()
+    kern_ms = sorted(e0.elapsed_time(e1) for e0, e1 in evs)
+    kern_avg_ms = sum(kern_ms) / len(kern_ms)
+
+    tflops = flops / (wall_ms * 1e-3) / 1e12
+    kern_tflops = flops / (kern_avg_ms * 1e-3) / 1e12
+    alg_bytes = inputs.algorithmic_bytes(cfg)
+
+    out = {
+        "metric": "fp8_attention_fwd_tflops",
+        "value": round(tflops, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "fp8_e4m3",
+        "data": "synthetic",
+        "config": {
+            "workload": f"{args.workload}: B={cfg['B']} H={cfg['H']} N={cfg['N']} d={cfg['d']} "
+                        f"{'causal' if causal else 'non-causal'}, e4m3 q/k/v ~ {cfg['dist']}, fp16 O, scale=1/sqrt(d)",
+            "flops_per_step": flops,
+            "pct_fp8_mfma_peak": round(100.0 * tflops / FP8_MFMA_PEAK_TFLOPS, 2),
+            "algorithmic_hbm_gbps": round(alg_bytes / (kern_avg_ms * 1e-3) / 1e9, 1),
+            "kv_block": fa.query(fa.FA8_QUERY_KV_BLOCK),
+        },
+        "roofline": {
+            "bound": "mfma",
+            "achieved": round(kern_tflops, 2),
+            "peak": FP8_MFMA_PEAK_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": round(kern_tflops / FP8_MFMA_PEAK_TFLOPS, 4),
+            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+            "kernel_ms_avg": round(kern_avg_ms, 5),
+            "kernel_ms_min": round(kern_ms[0], 5),
+            "kernel_ms_median": round(kern_ms[len(kern_ms) // 2], 5),
+        },
+    }
+
+    if not args.no_cpu_baseline:
+        # The reference's CPU-runnable path (naive attention, reference test.py:25-33) restated in oracle/ and timed
+        # on this machine's host cores, on the first heads of the same workload.
+        from oracle.naive_attention import naive_attention_cpu
+        cores = os.cpu_count() or 1
+        threads = min(cores, 16)
+        torch.set_num_threads(threads)
+        naive_attention_cpu(q8, k8, v8, scale, causal, heads_limit=1)  # warm-up, also sizes the sample
+        t0 = time.perf_counter()
+        naive_attention_cpu(q8, k8, v8, scale, causal, heads_limit=1)
+        per_head = time.perf_counter() - t0
+        n_heads_total = cfg["B"] * cfg["H"]
+        n = max(1, min(n_heads_total, int(args.cpu_seconds / max(per_head, 1e-6))))
+        t0 = time.perf_counter()
+        naive_attention_cpu(q8, k8, v8, scale, causal, heads_limit=n)
+        cpu_s = time.perf_counter() - t0
+        cpu_tflops = flops * (n / n_heads_total) / cpu_s / 1e12
+        out["cpu_baseline"] = {
+            "value": round(cpu_tflops, 4),
+            "unit": "TFLOP/s",
+            "cores": threads,
+            "kind": "port",
+            "sample": f"first {n} of {n_heads_total} (batch*head) slices of the same workload, {cpu_s:.2f} s, "
+                      f"torch CPU naive attention with P re-quantised to e4m3",
+        }
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

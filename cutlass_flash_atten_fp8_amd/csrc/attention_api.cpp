@@ -10,8 +10,8 @@
 //   * O is fp16 by default; `out_dtype=torch.float8_e4m3fn` gives the reference's fp8 O (:656);
 //   * the kernel runs on torch's current stream and the call does not synchronise the device (:661-665);
 //   * bad arguments and HIP errors raise RuntimeError instead of printf + exit (include/attention_api.cuh:20-29).
-#include <c10/hip/HIPGuard.h>
-#include <c10/hip/HIPStream.h>
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <torch/extension.h>
 
 #include <vector>
@@ -78,8 +78,9 @@ std::vector<torch::Tensor> flash_attention_v2_cutlass(torch::Tensor q, torch::Te
   p.v_batch_stride = v.stride(0); p.v_head_stride = v.stride(1); p.v_row_stride = v.stride(2);
   p.o_batch_stride = out.stride(0); p.o_head_stride = out.stride(1); p.o_row_stride = out.stride(2);
 
-  const c10::hip::HIPGuard device_guard(q.device());
-  const hipStream_t stream = c10::hip::getCurrentHIPStream(q.device().index()).stream();
+  // PyTorch-ROCm presents HIP devices under the "cuda" device type; these are its guard and stream for them.
+  const c10::hip::HIPGuardMasqueradingAsCUDA device_guard(q.device());
+  const hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(q.device().index()).stream();
   const int rc = fa8_fwd(&p, (void*)stream);
   TORCH_CHECK(rc == FA8_OK, "flash_attention_v2_cutlass: ", fa8_error_string(rc), " (code ", rc, ")");
   return {out};

@@ -24,6 +24,7 @@
 
 #include <cmath>
 #include <cstdint>
+#include <type_traits>
 
 #include "fa8_api.h"
 
@@ -99,12 +100,15 @@ __device__ __forceinline__ void tile_slot_decode(int slot, int& row, int& chunk)
 typedef unsigned v2u __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ float lane32_max(float x) {
   const v2u r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+  return __builtin_fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
 }
 __device__ __forceinline__ float lane32_sum(float x) {
   const v2u r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
+
+// max of three floats; the compiler fuses the pair into one v_max3_f32.
+__device__ __forceinline__ float max3(float a, float b, float c) { return __builtin_fmaxf(__builtin_fmaxf(a, b), c); }
 
 template <bool E5M2>
 __device__ __forceinline__ v16f mfma_fp8(const v8i& a, const v8i& b, const v16f& c) {
@@ -116,7 +120,7 @@ __device__ __forceinline__ v16f mfma_fp8(const v8i& a, const v8i& b, const v16f&
 
 template <bool E5M2>
 __device__ __forceinline__ int pack4_fp8(float a, float b, float c, float d) {
-  int r = 0;
+  int r = __float_as_int(a);  // any value: both 16-bit halves are overwritten below
   if constexpr (E5M2) {
     r = __builtin_amdgcn_cvt_pk_bf8_f32(a, b, r, false);
     r = __builtin_amdgcn_cvt_pk_bf8_f32(c, d, r, true);
@@ -148,11 +152,15 @@ template <int D, bool CAUSAL, bool E5M2, int OUT>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3))) void fa8_fwd_kernel(
     const KernelArgs a) {
   constexpr int kTileBytes = kKvBlock * D;      // one K or V tile
-  constexpr int kStageBytes = 2 * kTileBytes;   // K tile then V tile
   constexpr int kPasses = kTileBytes / (kThreads * 16);
   constexpr int kKSteps = D / 64;  // MFMA k-steps over the head dim for S^T
   constexpr int kMTiles = D / 32;  // 32-row tiles of O^T
-  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  // One LDS object per (stage, operand): the compiler then knows that the asynchronous HBM -> LDS copy into one
+  // stage cannot alias the reads of the other stage and does not wait for the copy before those reads.
+  __shared__ __attribute__((aligned(1024))) uint8_t k_lds0[kTileBytes];
+  __shared__ __attribute__((aligned(1024))) uint8_t k_lds1[kTileBytes];
+  __shared__ __attribute__((aligned(1024))) uint8_t v_lds0[kTileBytes];
+  __shared__ __attribute__((aligned(1024))) uint8_t v_lds1[kTileBytes];
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int qn = lane & 31, h = lane >> 5;
@@ -196,9 +204,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3))) v
     v_col[p] = ch * 16;
   }
   const int kv_last = a.seqlen_k - 1;
-  auto issue_tile = [&](int j, int stage) {
-    uint8_t* kb = smem + stage * kStageBytes;
-    uint8_t* vb = kb + kTileBytes;
+  // Start the asynchronous copy of KV block j into the LDS buffers kb / vb.
+  auto issue_tile = [&](int j, uint8_t* kb, uint8_t* vb) __attribute__((always_inline)) {
     const int kv0 = j * kKvBlock;
 #pragma unroll
     for (int p = 0; p < kPasses; ++p) {
@@ -211,8 +218,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3))) v
   };
 
   // ---- per-lane LDS read offsets ----
-  // K fragment (A operand of S^T): LDS row 32t + qn... the lane's row index inside the 32-row MFMA tile is
-  // lane % 32 and its k-group lane / 32; chunks 4ks+2h and 4ks+2h+1 of that row.
+  // K fragment (A operand of S^T): the lane's row inside the 32-row MFMA tile is lane % 32 and its k-group
+  // lane / 32: chunks 4ks+2h and 4ks+2h+1 of LDS row 32t + lane % 32.
   int k_off[kKSteps][2];
 #pragma unroll
   for (int ks = 0; ks < kKSteps; ++ks)
@@ -230,6 +237,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3))) v
 
   const int n_tiles = CAUSAL ? (min(a.seqlen_k, q0 + kQBlock) + kKvBlock - 1) / kKvBlock
                              : (a.seqlen_k + kKvBlock - 1) / kKvBlock;
+  // Leading blocks that need no mask for any row of the workgroup: they end at or before the first query row
+  // (causal) and inside the kv range.  They are processed in pairs by the mask-free copy of the loop body.
+  const int n_plain = (CAUSAL ? min(q0, a.seqlen_k) : a.seqlen_k) / kKvBlock;
 
   v16f o_acc[kMTiles];
 #pragma unroll
@@ -239,96 +249,108 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3))) v
   float m_run = -INFINITY;  // running row max of raw S (both half-lanes of a query hold the same value)
   float l_run = 0.f;        // this lane's share of the running row sum
 
-  issue_tile(0, 0);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __syncthreads();
-
-  for (int j = 0; j < n_tiles; ++j) {
-    if (j + 1 < n_tiles) issue_tile(j + 1, (j + 1) & 1);
-    const uint8_t* kb = smem + (j & 1) * kStageBytes;
-    const uint8_t* vb = kb + kTileBytes;
+  // S^T, online softmax and PV for KV block j held in kb / vb.
+  auto compute_tile = [&](int j, const uint8_t* kb, const uint8_t* vb, auto masked_c) __attribute__((always_inline)) {
+    constexpr bool kMasked = decltype(masked_c)::value;
     const int kv0 = j * kKvBlock;
-    // A wavefront whose 32 query rows all lie before this kv block has nothing to add (causal).
-    const bool active = !CAUSAL || (kv0 <= q_wave0 + kQWave - 1);
-    if (active) {
-      // ---- S^T = K Q^T : two 32(kv) x 32(q) sub-tiles ----
-      v16f s[2];
+    // ---- S^T = K Q^T : two 32(kv) x 32(q) sub-tiles ----
+    v16f s[2];
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
+    for (int t = 0; t < 2; ++t) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) s[t][i] = 0.f;
+      for (int i = 0; i < 16; ++i) s[t][i] = 0.f;
 #pragma unroll
-        for (int ks = 0; ks < kKSteps; ++ks) {
-          const v4i lo = *LDS_PTR(const v4i, kb + t * kSubTileStride + k_off[ks][0]);
-          const v4i hi = *LDS_PTR(const v4i, kb + t * kSubTileStride + k_off[ks][1]);
-          const v8i kf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-          s[t] = mfma_fp8<E5M2>(kf, qf[ks], s[t]);
-        }
-      }
-      // ---- causal / tail mask: register i of sub-tile t is kv row kv0 + 32h + 16t + i ----
-      const int kv_limit = CAUSAL ? min(q_row, kv_last) : kv_last;  // last kv this query attends to
-      const int wave_limit = CAUSAL ? min(q_wave0, kv_last) : kv_last;
-      const bool need_mask = kv0 + kKvBlock - 1 > wave_limit;
-      if (need_mask) {
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-          for (int i = 0; i < 16; ++i)
-            if (kv0 + 32 * h + 16 * t + i > kv_limit) s[t][i] = -INFINITY;
-      }
-      // ---- online softmax (reference softmax_rescale_o, csrc/flash_attention.cu:233-273) ----
-      float mloc = fmaxf(s[0][0], s[1][0]);
-#pragma unroll
-      for (int i = 1; i < 16; ++i) mloc = fmaxf(mloc, fmaxf(s[0][i], s[1][i]));
-      mloc = lane32_max(mloc);
-      const float m_new = fmaxf(m_run, mloc);
-      if (__any(m_new != m_run)) {
-        const float alpha = (m_run == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((m_run - m_new) * c);
-        l_run *= alpha;
-#pragma unroll
-        for (int mt = 0; mt < kMTiles; ++mt)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) o_acc[mt][i] *= alpha;
-        m_run = m_new;
-      }
-      const float mc = (m_new == -INFINITY) ? 0.f : m_new * c;
-      float sum0 = 0.f, sum1 = 0.f;
-      v8i p8;
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) s[t][i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][i], c, -mc));
-        if (need_mask) {
-          // a masked logit is -inf; force its weight to 0 even when scale <= 0 would give NaN or 1
-#pragma unroll
-          for (int i = 0; i < 16; ++i)
-            if (kv0 + 32 * h + 16 * t + i > kv_limit) s[t][i] = 0.f;
-        }
-#pragma unroll
-        for (int i = 0; i < 16; i += 2) {
-          sum0 += s[t][i];
-          sum1 += s[t][i + 1];
-        }
-#pragma unroll
-        for (int w = 0; w < 4; ++w)
-          p8[4 * t + w] = pack4_fp8<E5M2>(s[t][4 * w], s[t][4 * w + 1], s[t][4 * w + 2], s[t][4 * w + 3]);
-      }
-      l_run += sum0 + sum1;
-      // ---- O^T += V^T P^T ----
-#pragma unroll
-      for (int mt = 0; mt < kMTiles; ++mt) {
-        v8i vf;
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const v2i r = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_PTR(v2i, vb + v_off[mt] + g * kTrStride));
-          vf[2 * g] = r[0];
-          vf[2 * g + 1] = r[1];
-        }
-        o_acc[mt] = mfma_fp8<E5M2>(vf, p8, o_acc[mt]);
+      for (int ks = 0; ks < kKSteps; ++ks) {
+        const v4i lo = *LDS_PTR(const v4i, kb + t * kSubTileStride + k_off[ks][0]);
+        const v4i hi = *LDS_PTR(const v4i, kb + t * kSubTileStride + k_off[ks][1]);
+        const v8i kf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        s[t] = mfma_fp8<E5M2>(kf, qf[ks], s[t]);
       }
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
+    // ---- causal / tail mask: register i of sub-tile t is kv row kv0 + 32h + 16t + i ----
+    const int kv_limit = CAUSAL ? min(q_row, kv_last) : kv_last;  // last kv this query attends to
+    if constexpr (kMasked) {
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+          if (kv0 + 32 * h + 16 * t + i > kv_limit) s[t][i] = -INFINITY;
+    }
+    // ---- online softmax (reference softmax_rescale_o, csrc/flash_attention.cu:233-273) ----
+    float mx[4] = {m_run, m_run, m_run, m_run};  // four independent chains
+#pragma unroll
+    for (int i = 0; i < 16; ++i) mx[i & 3] = max3(mx[i & 3], s[0][i], s[1][i]);
+    const float m_new = lane32_max(max3(max3(mx[0], mx[1], mx[2]), mx[3], mx[3]));  // same in both half-lanes
+    if (__any(m_new != m_run)) {
+      const float alpha = (m_run == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((m_run - m_new) * c);
+      l_run *= alpha;
+#pragma unroll
+      for (int mt = 0; mt < kMTiles; ++mt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o_acc[mt][i] *= alpha;
+      m_run = m_new;
+    }
+    const float mc = (m_new == -INFINITY) ? 0.f : m_new * c;
+    float sum0 = 0.f, sum1 = 0.f;
+    v8i p8;
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s[t][i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][i], c, -mc));
+      if constexpr (kMasked) {
+        // a masked logit is -inf; force its weight to 0 even when scale <= 0 would give NaN or 1
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+          if (kv0 + 32 * h + 16 * t + i > kv_limit) s[t][i] = 0.f;
+      }
+#pragma unroll
+      for (int i = 0; i < 16; i += 2) {
+        sum0 += s[t][i];
+        sum1 += s[t][i + 1];
+      }
+#pragma unroll
+      for (int w = 0; w < 4; ++w)
+        p8[4 * t + w] = pack4_fp8<E5M2>(s[t][4 * w], s[t][4 * w + 1], s[t][4 * w + 2], s[t][4 * w + 3]);
+    }
+    l_run += sum0 + sum1;
+    // ---- O^T += V^T P^T ----
+#pragma unroll
+    for (int mt = 0; mt < kMTiles; ++mt) {
+      v8i vf;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const v2i r = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_PTR(v2i, vb + v_off[mt] + g * kTrStride));
+        vf[2 * g] = r[0];
+        vf[2 * g + 1] = r[1];
+      }
+      o_acc[mt] = mfma_fp8<E5M2>(vf, p8, o_acc[mt]);
+    }
+  };
+  auto stage_sync = [&]() __attribute__((always_inline)) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this lane's share of the next block has landed in LDS
+    __syncthreads();                                   // everyone's has, and everyone is done reading this block
+  };
+
+  issue_tile(0, k_lds0, v_lds0);
+  stage_sync();
+  int j = 0;
+  // Mask-free blocks, two per trip so that each half reads one fixed LDS stage while the copy fills the other.
+  for (; j + 1 < n_plain; j += 2) {
+    issue_tile(j + 1, k_lds1, v_lds1);
+    compute_tile(j, k_lds0, v_lds0, std::false_type());
+    stage_sync();
+    if (j + 2 < n_tiles) issue_tile(j + 2, k_lds0, v_lds0);
+    compute_tile(j + 1, k_lds1, v_lds1, std::false_type());
+    stage_sync();
+  }
+  // The remaining blocks (an odd mask-free one, the blocks on the diagonal, the kv tail) take the masking copy.
+  for (; j < n_tiles; ++j) {
+    const bool odd = j & 1;
+    if (j + 1 < n_tiles) issue_tile(j + 1, odd ? k_lds0 : k_lds1, odd ? v_lds0 : v_lds1);
+    // a wavefront whose 32 query rows all lie before this kv block has nothing to add (causal)
+    if (!CAUSAL || j * kKvBlock <= q_wave0 + kQWave - 1)
+      compute_tile(j, odd ? k_lds1 : k_lds0, odd ? v_lds1 : v_lds0, std::true_type());
+    stage_sync();
   }
 
   // ---- epilogue: O / l, convert, store (reference csrc/flash_attention.cu:542-582) ----
@@ -367,9 +389,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3))) v
 
 template <int D, bool CAUSAL, bool E5M2, int OUT>
 int launch(const KernelArgs& a, hipStream_t stream) {
-  constexpr int lds_bytes = 2 * 2 * kKvBlock * D;
   const dim3 grid((unsigned)(a.bh_total * a.n_qblocks));
-  hipLaunchKernelGGL((fa8_fwd_kernel<D, CAUSAL, E5M2, OUT>), grid, dim3(kThreads), lds_bytes, stream, a);
+  hipLaunchKernelGGL((fa8_fwd_kernel<D, CAUSAL, E5M2, OUT>), grid, dim3(kThreads), 0, stream, a);
   return (int)hipGetLastError();
 }
 

@@ -1,0 +1,115 @@
+"""C-ABI boundary, CPU only: libfa8.so loads, exports every function include/fa8_api.h declares, and the host-side
+argument validation returns the documented codes without touching a GPU.  No compute entry point is called with
+arguments that would pass validation."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+import cutlass_flash_atten_fp8_amd as fa
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions():
+    names = []
+    for fn in os.listdir(os.path.join(ROOT, "include")):
+        if fn.endswith(".h"):
+            text = open(os.path.join(ROOT, "include", fn)).read()
+            text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+            names += re.findall(r"^\s*(?:const\s+)?(?:int|char\s*\*|void)\s*\*?\s*(fa8_\w+)\s*\(", text, flags=re.M)
+    return sorted(set(names))
+
+
+def test_header_declares_the_expected_entry_points():
+    assert declared_functions() == sorted(fa.FA8_EXPORTS)
+
+
+def test_library_exports_every_declared_symbol():
+    lib = ctypes.CDLL(fa.LIBFA8_PATH)
+    for name in declared_functions():
+        assert getattr(lib, name) is not None
+
+
+def test_query_values():
+    assert fa.query(fa.FA8_QUERY_VERSION) >= 1
+    assert fa.query(fa.FA8_QUERY_KV_BLOCK) in (64, 128)
+    assert fa.query(fa.FA8_QUERY_Q_BLOCK) % 32 == 0
+    assert fa.query(fa.FA8_QUERY_KV_ASCENDING) == 1
+    assert fa.query(fa.FA8_QUERY_THREADS) % 64 == 0
+    assert fa.query(12345) == -1
+    assert fa.error_string(0) == "ok"
+    assert "head_dim" in fa.error_string(-3)
+    assert fa.error_string(-999)
+
+
+def cpu_tensors(n=64, d=64, dtype=torch.float8_e4m3fn, b=1, h=2):
+    q = torch.zeros((b, h, n, d), dtype=torch.float32).to(dtype)
+    return q, q.clone(), q.clone(), torch.zeros((b, h, n, d), dtype=torch.float16)
+
+
+def validate(p):
+    return fa.lib().fa8_fwd_validate(ctypes.byref(p))
+
+
+def test_validate_accepts_a_plain_problem():
+    q, k, v, o = cpu_tensors()
+    assert validate(fa.make_params(q, k, v, o, False, 0.125)) == 0
+    assert validate(fa.make_params(q, k, v, o, True, 0.125)) == 0
+    o8 = torch.zeros(o.shape, dtype=torch.float32).to(torch.float8_e4m3fn)
+    assert validate(fa.make_params(q, k, v, o8, False, 0.125)) == 0
+
+
+def test_validate_rejects_bad_arguments():
+    q, k, v, o = cpu_tensors()
+    assert fa.lib().fa8_fwd_validate(None) == -1
+    p = fa.make_params(q, k, v, o, False, 0.125); p.q = None
+    assert validate(p) == -1
+    p = fa.make_params(q, k, v, o, False, 0.125); p.seqlen_k = 0
+    assert validate(p) == -2
+    p = fa.make_params(q, k, v, o, True, 0.125); p.seqlen_k = 32
+    assert validate(p) == -2  # causal needs seqlen_q == seqlen_k
+    for d in (32, 96, 256):
+        q2, k2, v2, o2 = cpu_tensors(d=d)
+        assert validate(fa.make_params(q2, k2, v2, o2, False, 0.125)) == -3
+    p = fa.make_params(q, k, v, o, False, 0.125); p.k_row_stride = 32
+    assert validate(p) == -4
+    p = fa.make_params(q, k, v, o, False, 0.125); p.k_row_stride = 72
+    assert validate(p) == -5
+    p = fa.make_params(q, k, v, o, False, 0.125); p.q = p.q + 4
+    assert validate(p) == -5
+    p = fa.make_params(q, k, v, o, False, 0.125); p.in_dtype = 7
+    assert validate(p) == -6
+    p = fa.make_params(q, k, v, o, False, 0.125); p.out_dtype = 9
+    assert validate(p) == -6
+    for bad in (float("nan"), float("inf")):
+        assert validate(fa.make_params(q, k, v, o, False, bad)) == -8
+
+
+def test_fa8_fwd_rejects_before_any_gpu_work():
+    # invalid arguments must come back as negative codes even on a machine without a GPU
+    q, k, v, o = cpu_tensors(d=96)
+    p = fa.make_params(q, k, v, o, False, 0.125)
+    assert fa.lib().fa8_fwd(ctypes.byref(p), None) == -3
+
+
+def test_python_operator_mirrors_reference_errors():
+    q, k, v, _ = cpu_tensors()
+    with pytest.raises(RuntimeError, match="GPU tensor"):
+        fa.flash_attention_v2_cutlass(q, k, v, False, 0.125)
+    with pytest.raises(TypeError):
+        fa.flash_attention_v2_cutlass(q, k, v)  # all five arguments are required, as in the reference binding
+
+
+def test_compiled_binding_mirrors_reference_errors():
+    ext = fa.load_extension()
+    import attention_cutlass_fp8
+    assert attention_cutlass_fp8 is ext
+    q, k, v, _ = cpu_tensors()
+    with pytest.raises(RuntimeError, match="GPU tensor"):
+        ext.flash_attention_v2_cutlass(q, k, v, False, 0.125)
+    with pytest.raises(TypeError):
+        ext.flash_attention_v2_cutlass(q, k, v)
+    assert ext.kv_block() == fa.query(fa.FA8_QUERY_KV_BLOCK)

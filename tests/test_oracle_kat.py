@@ -1,0 +1,213 @@
+"""Pins the CPU oracle (oracle/fa8_oracle.c) without the reference: closed-form known answers, invariants,
+a brute-force fp64 restatement on tiny inputs, equality with textbook softmax attention when the P quantisation is
+switched off, and agreement with an independent numpy restatement.  Each check is chosen so that a plausible
+mistake (row sum taken from the quantised P, a missing rescale, an off-by-one causal mask, a transposed operand,
+max over scaled instead of raw logits) fails it.
+"""
+import math
+
+import numpy as np
+import pytest
+
+from oracle import fa8_oracle as fo
+from oracle import np_restatement as nr
+
+
+def enc(x):
+    return nr.encode_rne_sat(np.asarray(x, dtype=np.float64))
+
+
+def dec(c):
+    return nr.decode(c)
+
+
+def rand_qkv(rng, shape, s=1.0):
+    return tuple(enc(rng.standard_normal(shape) * s) for _ in range(3))
+
+
+def test_causal_row0_is_v0_exactly():
+    rng = np.random.default_rng(1)
+    q, k, v = rand_qkv(rng, (2, 2, 70, 64))
+    o = fo.forward(q, k, v, 0.125, causal=True)
+    assert np.array_equal(o[:, :, 0, :].astype(np.float64), dec(v)[:, :, 0, :])
+
+
+def test_equal_keys_give_mean_of_v():
+    rng = np.random.default_rng(2)
+    q, k, v = rand_qkv(rng, (1, 2, 96, 64))
+    k[:] = k[:, :, :1, :]  # all keys identical -> every P is exactly 1.0 -> O = mean(V)
+    o = fo.forward(q, k, v, 0.3, out_dtype=fo.OUT_F32)
+    want = dec(v).mean(axis=2, keepdims=True)
+    assert np.allclose(o, np.broadcast_to(want, o.shape), rtol=0, atol=2e-6)
+    oc = fo.forward(q, k, v, 0.3, causal=True, out_dtype=fo.OUT_F32)
+    prefix = np.cumsum(dec(v), axis=2) / np.arange(1, 97)[None, None, :, None]
+    assert np.allclose(oc, prefix, rtol=0, atol=2e-6)
+
+
+def test_scale_zero_gives_mean_of_v():
+    rng = np.random.default_rng(3)
+    q, k, v = rand_qkv(rng, (1, 1, 130, 64))
+    o = fo.forward(q, k, v, 0.0, out_dtype=fo.OUT_F32)
+    assert np.allclose(o, np.broadcast_to(dec(v).mean(axis=2, keepdims=True), o.shape), rtol=0, atol=2e-6)
+    oc = fo.forward(q, k, v, 0.0, causal=True, out_dtype=fo.OUT_F32)
+    prefix = np.cumsum(dec(v), axis=2) / np.arange(1, 131)[None, None, :, None]
+    assert np.allclose(oc, prefix, rtol=0, atol=2e-6)
+
+
+def test_dominant_logit_selects_one_value_row():
+    d, n = 64, 200
+    q = np.zeros((1, 1, n, d)); k = np.zeros((1, 1, n, d))
+    q[..., 0] = 16.0
+    k[..., 0] = -16.0
+    sel = [(i * 37 + 11) % n for i in range(n)]
+    rng = np.random.default_rng(4)
+    v = rng.standard_normal((1, 1, n, d))
+    # every query has the same logits: -256 everywhere except +256 at column 133: a gap of 512 * scale >> 20
+    k[0, 0, 133, 0] = 16.0
+    o = fo.forward(enc(q), enc(k), enc(v), 1.0)
+    assert np.array_equal(o[0, 0].astype(np.float64), np.broadcast_to(dec(enc(v))[0, 0, 133], (n, d)))
+    del sel
+
+
+def test_constant_v_separates_fp32_row_sum_from_quantised_row_sum():
+    """V == c gives O = c * sum(P8) / sum(P): it equals c only if the denominator wrongly used the quantised P."""
+    rng = np.random.default_rng(5)
+    q, k, _ = rand_qkv(rng, (1, 1, 64, 64))
+    v = enc(np.full((1, 1, 64, 64), 1.5))
+    o = fo.forward(q, k, v, 0.125, out_dtype=fo.OUT_F32)[0, 0]
+    qf, kf = dec(q)[0, 0], dec(k)[0, 0]
+    s = qf @ kf.T
+    p = np.exp((s - s.max(axis=1, keepdims=True)) * 0.125)
+    p8 = dec(enc(p))
+    want = 1.5 * p8.sum(axis=1) / p.sum(axis=1)
+    assert np.allclose(o, want[:, None], rtol=2e-5, atol=0)
+    assert np.abs(want - 1.5).max() > 1e-3  # the case does discriminate
+
+
+def brute_force(q, k, v, scale, causal, bc):
+    """Scalar fp64 loops with explicit e4m3 rounding of P (tiny inputs only)."""
+    qf, kf, vf = dec(q), dec(k), dec(v)
+    B, H, n, d = qf.shape
+    out = np.zeros((B, H, n, d))
+    for b in range(B):
+        for h in range(H):
+            for i in range(n):
+                m, l, o = -math.inf, 0.0, np.zeros(d)
+                for j0 in range(0, n, bc):
+                    cols = [j for j in range(j0, min(j0 + bc, n)) if (not causal or j <= i)]
+                    if not cols:
+                        continue
+                    s = [sum(qf[b, h, i, x] * kf[b, h, j, x] for x in range(d)) for j in cols]
+                    m_new = max(m, max(s))
+                    alpha = 0.0 if m == -math.inf else math.exp((m - m_new) * scale)
+                    p = [math.exp((sj - m_new) * scale) for sj in s]
+                    l = l * alpha + sum(p)
+                    p8 = dec(enc(np.array(p)))
+                    o = o * alpha + sum(p8[t] * vf[b, h, j] for t, j in enumerate(cols))
+                    m = m_new
+                out[b, h, i] = o / l
+    return out
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("bc", [2, 3, 8])
+def test_brute_force_tiny(causal, bc):
+    rng = np.random.default_rng(10 + bc)
+    q, k, v = rand_qkv(rng, (1, 2, 8, 64))
+    want = brute_force(q, k, v, 0.125, causal, bc)
+    got = fo.forward(q, k, v, 0.125, causal=causal, kv_block=bc, out_dtype=fo.OUT_F32)
+    # fp32 vs fp64 arithmetic can flip the rounding of a P that sits on a boundary: allow isolated flips
+    err = np.abs(got - want)
+    assert np.median(err) < 1e-6
+    assert (err > 1e-4).mean() < 0.02
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("bc", [16, 64, 100, 1000])
+def test_without_quantisation_equals_textbook_attention(causal, bc):
+    rng = np.random.default_rng(20)
+    q, k, v = rand_qkv(rng, (2, 2, 257, 64))
+    got = fo.forward(q, k, v, 0.125, causal=causal, kv_block=bc, quantize_p=False, out_dtype=fo.OUT_F32)
+    want = fo.attention_f64(q, k, v, 0.125, causal=causal)
+    assert np.abs(got - want).max() < 5e-6
+    # and the fp64 attention itself against a direct numpy softmax
+    qf, kf, vf = dec(q), dec(k), dec(v)
+    s = np.einsum("bhid,bhjd->bhij", qf, kf) * 0.125
+    if causal:
+        s = np.where(np.tril(np.ones((257, 257), dtype=bool)), s, -np.inf)
+    p = np.exp(s - s.max(axis=-1, keepdims=True))
+    ref = np.einsum("bhij,bhjd->bhid", p / p.sum(axis=-1, keepdims=True), vf)
+    assert np.abs(want - ref).max() < 1e-12
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("shape,bc", [((1, 2, 128, 64), 64), ((2, 1, 200, 128), 64), ((1, 1, 300, 64), 128)])
+def test_c_oracle_matches_numpy_restatement(shape, bc, causal):
+    rng = np.random.default_rng(30)
+    q, k, v = rand_qkv(rng, shape)
+    scale = 1 / math.sqrt(shape[-1])
+    a = fo.forward(q, k, v, scale, causal=causal, kv_block=bc, out_dtype=fo.OUT_F32)
+    b = nr.forward(q, k, v, scale, causal=causal, kv_block=bc, out="f32")
+    err = np.abs(a - b)
+    # two fp32 implementations with different summation orders: identical up to isolated P rounding flips
+    assert np.median(err) < 1e-6
+    assert err.mean() < 2e-4 and (err > 2e-3).mean() < 0.02
+
+
+def test_kv_block_changes_the_result_only_through_quantisation():
+    rng = np.random.default_rng(40)
+    q, k, v = rand_qkv(rng, (1, 2, 512, 64))
+    a = fo.forward(q, k, v, 0.125, kv_block=64, out_dtype=fo.OUT_F32)
+    b = fo.forward(q, k, v, 0.125, kv_block=128, out_dtype=fo.OUT_F32)
+    d = np.abs(a - b)
+    assert 1e-5 < d.mean() < 2e-3  # block size matters (running max P is quantised against) but stays in budget
+    a0 = fo.forward(q, k, v, 0.125, kv_block=64, quantize_p=False, out_dtype=fo.OUT_F32)
+    b0 = fo.forward(q, k, v, 0.125, kv_block=128, quantize_p=False, out_dtype=fo.OUT_F32)
+    assert np.abs(a0 - b0).max() < 5e-6
+
+
+def test_causal_rows_ignore_future_keys_and_values():
+    rng = np.random.default_rng(50)
+    q, k, v = rand_qkv(rng, (1, 1, 160, 64))
+    a = fo.forward(q, k, v, 0.125, causal=True)
+    k2, v2 = k.copy(), v.copy()
+    k2[:, :, 100:, :] = enc(rng.standard_normal((1, 1, 60, 64)) * 3)
+    v2[:, :, 100:, :] = enc(rng.standard_normal((1, 1, 60, 64)) * 3)
+    b = fo.forward(q, k2, v2, 0.125, causal=True)
+    assert np.array_equal(a[:, :, :100].view(np.uint16), b[:, :, :100].view(np.uint16))
+    assert not np.array_equal(a[:, :, 100:].view(np.uint16), b[:, :, 100:].view(np.uint16))
+
+
+def test_row_subset_and_transposed_v_and_outputs():
+    rng = np.random.default_rng(60)
+    q, k, v = rand_qkv(rng, (2, 2, 150, 64))
+    full = fo.forward(q, k, v, 0.125, causal=True)
+    rows = np.array([0, 5, 64, 149], dtype=np.int32)
+    sub = fo.forward(q, k, v, 0.125, causal=True, rows=rows)
+    assert np.array_equal(sub.view(np.uint16), full[:, :, rows].view(np.uint16))
+    vt = np.ascontiguousarray(v.transpose(0, 1, 3, 2))
+    assert np.array_equal(fo.forward(q, k, vt, 0.125, causal=True, v_transposed=True).view(np.uint16), full.view(np.uint16))
+    f32 = fo.forward(q, k, v, 0.125, causal=True, out_dtype=fo.OUT_F32)
+    with np.errstate(over="ignore"):
+        assert np.array_equal(f32.astype(np.float16).view(np.uint16), full.view(np.uint16))
+    o8 = fo.forward(q, k, v, 0.125, causal=True, out_dtype=fo.OUT_E4M3)
+    assert np.array_equal(o8, enc(f32))
+
+
+def test_exp2_form_is_the_same_pipeline():
+    rng = np.random.default_rng(70)
+    q, k, v = rand_qkv(rng, (1, 2, 1024, 128))
+    a = fo.forward(q, k, v, 1 / math.sqrt(128), out_dtype=fo.OUT_F32)
+    b = fo.forward(q, k, v, 1 / math.sqrt(128), exp2_form=True, out_dtype=fo.OUT_F32)
+    d = np.abs(a - b)
+    assert d.max() < 2e-3 and d.mean() < 1e-5
+
+
+def test_flip_allowance_is_zero_without_near_ties_and_bounded():
+    rng = np.random.default_rng(80)
+    q, k, v = rand_qkv(rng, (1, 2, 256, 64))
+    _, allow0 = fo.forward(q, k, v, 0.125, logit_rel_err=0.0)
+    assert allow0.max() == 0.0
+    _, allow = fo.forward(q, k, v, 0.125, causal=True, logit_rel_err=2e-5)
+    assert (allow >= 0).all() and allow[:, :, 0].max() == 0.0  # row 0 has the single P = 1.0: never near a boundary
+    assert (allow > 0.02).mean() < 0.05
