@@ -28,6 +28,10 @@
 
 #include "fa8_api.h"
 
+#ifndef FA8_WAVES_PER_EU
+#define FA8_WAVES_PER_EU 3  // at most 168 VGPRs per lane
+#endif
+
 namespace {
 
 typedef int v2i __attribute__((ext_vector_type(2)));
@@ -120,7 +124,8 @@ __device__ __forceinline__ v16f mfma_fp8(const v8i& a, const v8i& b, const v16f&
 
 template <bool E5M2>
 __device__ __forceinline__ int pack4_fp8(float a, float b, float c, float d) {
-  int r = __float_as_int(a);  // any value: both 16-bit halves are overwritten below
+  int r;
+  asm("" : "=v"(r));  // any value will do (both 16-bit halves are overwritten below): define r without an instruction
   if constexpr (E5M2) {
     r = __builtin_amdgcn_cvt_pk_bf8_f32(a, b, r, false);
     r = __builtin_amdgcn_cvt_pk_bf8_f32(c, d, r, true);
@@ -149,8 +154,9 @@ __device__ __forceinline__ void decode_block(const KernelArgs& a, int id, int& b
 }
 
 template <int D, bool CAUSAL, bool E5M2, int OUT>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3))) void fa8_fwd_kernel(
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WAVES_PER_EU))) void fa8_fwd_kernel(
     const KernelArgs a) {
+#if defined(__HIP_DEVICE_COMPILE__)  // the body uses device-only types (buffer resources); the host pass only needs the stub
   constexpr int kTileBytes = kKvBlock * D;      // one K or V tile
   constexpr int kPasses = kTileBytes / (kThreads * 16);
   constexpr int kKSteps = D / 64;  // MFMA k-steps over the head dim for S^T
@@ -159,10 +165,13 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3))) v
   // stage cannot alias the reads of the other stage and does not wait for the copy before those reads.
   __shared__ __attribute__((aligned(1024))) uint8_t k_lds0[kTileBytes];
   __shared__ __attribute__((aligned(1024))) uint8_t k_lds1[kTileBytes];
+  __shared__ __attribute__((aligned(1024))) uint8_t k_lds2[kTileBytes];
   __shared__ __attribute__((aligned(1024))) uint8_t v_lds0[kTileBytes];
   __shared__ __attribute__((aligned(1024))) uint8_t v_lds1[kTileBytes];
+  __shared__ __attribute__((aligned(1024))) uint8_t v_lds2[kTileBytes];
 
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keep it (and all it feeds) in scalar registers
   const int qn = lane & 31, h = lane >> 5;
 
   int bh, qb;
@@ -189,31 +198,35 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3))) v
     }
   }
 
-  // ---- per-lane constants of the HBM -> LDS copy ----
-  // In pass p wavefront w fills LDS bytes [(4p+w)*1024, +1024) of the tile, lane l the 16 bytes at +16l.
-  int k_row[kPasses], k_col[kPasses], v_row[kPasses], v_col[kPasses];
+  // ---- HBM -> LDS copy: buffer_load_dwordx4 ... lds ----
+  // In pass p wavefront w fills LDS bytes [(4p+w)*1024, +1024) of the tile, lane l the 16 bytes at +16l; which
+  // (kv row, 16-byte chunk) belongs there follows from the swizzle.  The source address is the head's base (buffer
+  // resource) + a per-lane byte offset that never changes (VGPR) + the block's byte offset (SGPR): no vector ALU
+  // work per block.  The resource ends with the last kv row, so rows past the end of a ragged last block read 0.
+  unsigned k_src[kPasses], v_src[kPasses];
 #pragma unroll
   for (int p = 0; p < kPasses; ++p) {
     const int slot = (p * 4 + wave) * 64 + lane;
     int r, ch;
     tile_slot_decode<D, false>(slot, r, ch);
-    k_row[p] = kv_of_lds_row(r);
-    k_col[p] = ch * 16;
+    k_src[p] = (unsigned)(kv_of_lds_row(r) * (int)a.k_rs + ch * 16);
     tile_slot_decode<D, true>(slot, r, ch);
-    v_row[p] = r;
-    v_col[p] = ch * 16;
+    v_src[p] = (unsigned)(r * (int)a.v_rs + ch * 16);
   }
   const int kv_last = a.seqlen_k - 1;
+  constexpr int kRsrcFlags = 0x00020000;  // raw buffer, 32-bit data format
+  const __amdgpu_buffer_rsrc_t k_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void*)kp, 0, (int)(kv_last * a.k_rs + D), kRsrcFlags);
+  const __amdgpu_buffer_rsrc_t v_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void*)vp, 0, (int)(kv_last * a.v_rs + D), kRsrcFlags);
   // Start the asynchronous copy of KV block j into the LDS buffers kb / vb.
   auto issue_tile = [&](int j, uint8_t* kb, uint8_t* vb) __attribute__((always_inline)) {
-    const int kv0 = j * kKvBlock;
+    const int k_base = j * kKvBlock * (int)a.k_rs, v_base = j * kKvBlock * (int)a.v_rs;
 #pragma unroll
     for (int p = 0; p < kPasses; ++p) {
       const int seg = (p * 4 + wave) * 1024;
-      const uint8_t* ks = kp + (long long)min(kv0 + k_row[p], kv_last) * a.k_rs + k_col[p];
-      const uint8_t* vs = vp + (long long)min(kv0 + v_row[p], kv_last) * a.v_rs + v_col[p];
-      __builtin_amdgcn_global_load_lds(GLOBAL_PTR(const void, ks), LDS_PTR(void, kb + seg), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds(GLOBAL_PTR(const void, vs), LDS_PTR(void, vb + seg), 16, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, LDS_PTR(void, kb + seg), 16, k_src[p], k_base, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(v_rsrc, LDS_PTR(void, vb + seg), 16, v_src[p], v_base, 0, 0);
     }
   };
 
@@ -277,9 +290,11 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3))) v
           if (kv0 + 32 * h + 16 * t + i > kv_limit) s[t][i] = -INFINITY;
     }
     // ---- online softmax (reference softmax_rescale_o, csrc/flash_attention.cu:233-273) ----
-    float mx[4] = {m_run, m_run, m_run, m_run};  // four independent chains
+    float mx[4] = {m_run, m_run, m_run, m_run};  // four independent chains; sub-tile 0 first (it is ready first)
 #pragma unroll
-    for (int i = 0; i < 16; ++i) mx[i & 3] = max3(mx[i & 3], s[0][i], s[1][i]);
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int i = 0; i < 16; i += 2) mx[(i >> 1) & 3] = max3(mx[(i >> 1) & 3], s[t][i], s[t][i + 1]);
     const float m_new = lane32_max(max3(max3(mx[0], mx[1], mx[2]), mx[3], mx[3]));  // same in both half-lanes
     if (__any(m_new != m_run)) {
       const float alpha = (m_run == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((m_run - m_new) * c);
@@ -313,9 +328,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3))) v
         p8[4 * t + w] = pack4_fp8<E5M2>(s[t][4 * w], s[t][4 * w + 1], s[t][4 * w + 2], s[t][4 * w + 3]);
     }
     l_run += sum0 + sum1;
-    // ---- O^T += V^T P^T ----
-#pragma unroll
-    for (int mt = 0; mt < kMTiles; ++mt) {
+    // ---- O^T += V^T P^T : the V^T fragment of tile mt+1 is fetched while the MFMA of tile mt runs ----
+    auto load_vf = [&](int mt) __attribute__((always_inline)) {
       v8i vf;
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
@@ -323,34 +337,62 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3))) v
         vf[2 * g] = r[0];
         vf[2 * g + 1] = r[1];
       }
-      o_acc[mt] = mfma_fp8<E5M2>(vf, p8, o_acc[mt]);
+      return vf;
+    };
+    v8i vf_cur = load_vf(0);
+#pragma unroll
+    for (int mt = 0; mt < kMTiles; ++mt) {
+      v8i vf_next;
+      if (mt + 1 < kMTiles) vf_next = load_vf(mt + 1);
+      o_acc[mt] = mfma_fp8<E5M2>(vf_cur, p8, o_acc[mt]);
+      if (mt + 1 < kMTiles) vf_cur = vf_next;
     }
   };
-  auto stage_sync = [&]() __attribute__((always_inline)) {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this lane's share of the next block has landed in LDS
-    __syncthreads();                                   // everyone's has, and everyone is done reading this block
+  // Three LDS stages, copies issued two KV blocks ahead.  At the end of the step for block j the copy of block
+  // j+1 (issued one step earlier) must have landed while the copy of block j+2 (issued in this step: kLoadsPerTile
+  // loads per lane) may stay in flight; vmcnt counts this lane's loads in issue order.  The barrier then tells every
+  // wavefront that all shares of block j+1 are in LDS and that block j's stage may be overwritten.  It is a bare
+  // s_barrier: __syncthreads() would also wait for the copy that is meant to stay in flight.
+  constexpr int kLoadsPerTile = 2 * kPasses;
+  auto stage_sync = [&](bool next_in_flight) __attribute__((always_inline)) {
+    // s_waitcnt immediate (gfx9 layout): vmcnt[3:0], expcnt[6:4] = 7 and lgkmcnt[11:8] = 15 (no wait on those)
+    if (next_in_flight)
+      __builtin_amdgcn_s_waitcnt(0x0F70 | kLoadsPerTile);
+    else
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+    __builtin_amdgcn_s_barrier();
   };
+  static_assert(kLoadsPerTile < 16, "vmcnt immediate above");
 
   issue_tile(0, k_lds0, v_lds0);
-  stage_sync();
+  if (n_tiles > 1) issue_tile(1, k_lds1, v_lds1);
+  stage_sync(n_tiles > 1);
   int j = 0;
-  // Mask-free blocks, two per trip so that each half reads one fixed LDS stage while the copy fills the other.
-  for (; j + 1 < n_plain; j += 2) {
-    issue_tile(j + 1, k_lds1, v_lds1);
+  // Mask-free blocks, three per trip so that every third reads one fixed LDS stage (the compiler can then tell
+  // that the copies in flight go to other stages and need not be waited for before the reads).
+  // Inside this loop every copy is issued unconditionally (block j+4 exists), which lets the compiler see that each
+  // s_waitcnt below always leaves exactly one block in flight.
+  for (; j + 2 < n_plain && j + 4 < n_tiles; j += 3) {
+    issue_tile(j + 2, k_lds2, v_lds2);
     compute_tile(j, k_lds0, v_lds0, std::false_type());
-    stage_sync();
-    if (j + 2 < n_tiles) issue_tile(j + 2, k_lds0, v_lds0);
+    stage_sync(true);
+    issue_tile(j + 3, k_lds0, v_lds0);
     compute_tile(j + 1, k_lds1, v_lds1, std::false_type());
-    stage_sync();
+    stage_sync(true);
+    issue_tile(j + 4, k_lds1, v_lds1);
+    compute_tile(j + 2, k_lds2, v_lds2, std::false_type());
+    stage_sync(true);
   }
-  // The remaining blocks (an odd mask-free one, the blocks on the diagonal, the kv tail) take the masking copy.
+  // The remaining blocks (the last few mask-free ones, the blocks on the diagonal, the kv tail) take the masking copy.
   for (; j < n_tiles; ++j) {
-    const bool odd = j & 1;
-    if (j + 1 < n_tiles) issue_tile(j + 1, odd ? k_lds0 : k_lds1, odd ? v_lds0 : v_lds1);
+    const int st = j % 3, st2 = (j + 2) % 3;
+    if (j + 2 < n_tiles)
+      issue_tile(j + 2, st2 == 0 ? k_lds0 : (st2 == 1 ? k_lds1 : k_lds2), st2 == 0 ? v_lds0 : (st2 == 1 ? v_lds1 : v_lds2));
     // a wavefront whose 32 query rows all lie before this kv block has nothing to add (causal)
     if (!CAUSAL || j * kKvBlock <= q_wave0 + kQWave - 1)
-      compute_tile(j, odd ? k_lds1 : k_lds0, odd ? v_lds1 : v_lds0, std::true_type());
-    stage_sync();
+      compute_tile(j, st == 0 ? k_lds0 : (st == 1 ? k_lds1 : k_lds2), st == 0 ? v_lds0 : (st == 1 ? v_lds1 : v_lds2),
+                   std::true_type());
+    stage_sync(j + 2 < n_tiles);
   }
 
   // ---- epilogue: O / l, convert, store (reference csrc/flash_attention.cu:542-582) ----
@@ -385,6 +427,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3))) v
         }
     }
   }
+#endif  // __HIP_DEVICE_COMPILE__
 }
 
 template <int D, bool CAUSAL, bool E5M2, int OUT>
@@ -426,7 +469,6 @@ extern "C" int fa8_fwd_validate(const Fa8FwdParams* p) {
   if (!span_ok(p->k_row_stride, d) || !span_ok(p->k_head_stride, 1) || !span_ok(p->k_batch_stride, 1)) return FA8_ERR_STRIDE;
   if (!span_ok(p->v_row_stride, v_cols) || !span_ok(p->v_head_stride, 1) || !span_ok(p->v_batch_stride, 1)) return FA8_ERR_STRIDE;
   if (!span_ok(p->o_row_stride, d) || !span_ok(p->o_head_stride, 1) || !span_ok(p->o_batch_stride, 1)) return FA8_ERR_STRIDE;
-  (void)v_rows;
   // 16-byte vector loads of q/k/v rows, 8-byte (fp16) or 4-byte (fp8) vector stores of o
   const long long in_strides[] = {p->q_batch_stride, p->q_head_stride, p->q_row_stride, p->k_batch_stride, p->k_head_stride,
                                   p->k_row_stride,   p->v_batch_stride, p->v_head_stride, p->v_row_stride};
@@ -438,6 +480,8 @@ extern "C" int fa8_fwd_validate(const Fa8FwdParams* p) {
   for (long long s : o_strides)
     if ((s * o_elem) % 8 != 0) return FA8_ERR_ALIGN;
   if ((uintptr_t)p->o % 8 != 0) return FA8_ERR_ALIGN;
+  // the kernels address k and v of one head with 32-bit byte offsets
+  if ((long long)p->seqlen_k * p->k_row_stride > 0x7fffffffLL || v_rows * p->v_row_stride > 0x7fffffffLL) return FA8_ERR_SHAPE;
   if (p->v_layout == FA8_V_TRANSPOSED) return FA8_ERR_UNSUPPORTED;
   if (p->in_dtype == FA8_DTYPE_E5M2 && p->out_dtype == FA8_OUT_E4M3) return FA8_ERR_UNSUPPORTED;
   return FA8_OK;
