@@ -23,17 +23,20 @@ HBM_PEAK_GBPS = 8000.0
 
 # HBM bytes per launch of the headline workload read by rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), each scaled by
 # what the same counter reads for a plain copy kernel of known size; see profiles/.  None until measured.
-MEASURED_TRAFFIC_BYTES = {}
+MEASURED_TRAFFIC_BYTES = {"cfg3": 168.0e6}  # profiles/fa8_fwd_kernel_d128_cfg3_headline.md, section 3
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="cfg3", help="cfg1..cfg5 (cfg3 is the headline)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the baseline sample")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="run only a plain 256 MiB device-to-device copy (10 times): the known-size kernel that the "
+                         "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (the path shards over batch*heads with no communication; "
@@ -46,6 +49,14 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(3)
+    if args.copy_calibration:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda:0").fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(10):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_calibration_bytes_read": 256 << 20, "copy_calibration_bytes_written": 256 << 20, "launches": 10}))
+        return
     ext = fa.load_extension()  # raises if the native code has not been built: there is no fallback path
     cfg = inputs.CONFIGS[args.workload]
     scale = inputs.softmax_scale(cfg)
@@ -129,17 +140,19 @@ def main():
         per_head = time.perf_counter() - t0
         n_heads_total = cfg["B"] * cfg["H"]
         n = max(1, min(n_heads_total, int(args.cpu_seconds / max(per_head, 1e-6))))
+        reps = max(1, min(8, int(args.cpu_seconds / max(per_head * n, 1e-6))))  # small workloads: several passes
         t0 = time.perf_counter()
-        naive_attention_cpu(q8, k8, v8, scale, causal, heads_limit=n)
-        cpu_s = time.perf_counter() - t0
+        for _ in range(reps):
+            naive_attention_cpu(q8, k8, v8, scale, causal, heads_limit=n)
+        cpu_s = (time.perf_counter() - t0) / reps
         cpu_tflops = flops * (n / n_heads_total) / cpu_s / 1e12
         out["cpu_baseline"] = {
             "value": round(cpu_tflops, 4),
             "unit": "TFLOP/s",
             "cores": threads,
             "kind": "port",
-            "sample": f"first {n} of {n_heads_total} (batch*head) slices of the same workload, {cpu_s:.2f} s, "
-                      f"torch CPU naive attention with P re-quantised to e4m3",
+            "sample": f"first {n} of {n_heads_total} (batch*head) slices of the same workload, {reps} pass(es) of "
+                      f"{cpu_s:.2f} s, torch CPU naive attention with P re-quantised to e4m3",
         }
     print(json.dumps(out), flush=True)
 

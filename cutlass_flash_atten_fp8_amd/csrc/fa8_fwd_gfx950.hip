@@ -29,7 +29,7 @@
 #include "fa8_api.h"
 
 #ifndef FA8_WAVES_PER_EU
-#define FA8_WAVES_PER_EU 2  // at most 256 VGPRs per lane
+#define FA8_WAVES_PER_EU 3  // at most 168 VGPRs per lane
 #endif
 
 namespace {
@@ -104,7 +104,8 @@ __device__ __forceinline__ void tile_slot_decode(int slot, int& row, int& chunk)
 typedef unsigned v2u __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ float lane32_max(float x) {
   const v2u r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-  return __builtin_fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+  // median(a, b, +inf) = max(a, b) in one instruction (fmaxf would first quiet both operands)
+  return __builtin_amdgcn_fmed3f(__uint_as_float(r[0]), __uint_as_float(r[1]), INFINITY);
 }
 __device__ __forceinline__ float lane32_sum(float x) {
   const v2u r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
@@ -125,7 +126,7 @@ __device__ __forceinline__ v16f mfma_fp8(const v8i& a, const v8i& b, const v16f&
 template <bool E5M2>
 __device__ __forceinline__ int pack4_fp8(float a, float b, float c, float d) {
   int r;
-  asm("" : "=v"(r));  // any value will do (both 16-bit halves are overwritten below): define r without an instruction
+  asm volatile("" : "=v"(r));  // any value will do (both 16-bit halves are overwritten below): defines r, emits nothing
   if constexpr (E5M2) {
     r = __builtin_amdgcn_cvt_pk_bf8_f32(a, b, r, false);
     r = __builtin_amdgcn_cvt_pk_bf8_f32(c, d, r, true);
@@ -219,24 +220,14 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
       __builtin_amdgcn_make_buffer_rsrc((void*)kp, 0, (int)(kv_last * a.k_rs + D), kRsrcFlags);
   const __amdgpu_buffer_rsrc_t v_rsrc =
       __builtin_amdgcn_make_buffer_rsrc((void*)vp, 0, (int)(kv_last * a.v_rs + D), kRsrcFlags);
-  // KV block j travels HBM -> registers (fetch_tile: plain buffer loads, asynchronous, cheap to issue) -> LDS
-  // (commit_tile, one KV step later).  Loads that write LDS directly were measured to stall the issuing wavefront for
-  // most of the memory latency once several wavefronts per CU keep such loads in flight.
-  v4i stage_k[kPasses], stage_v[kPasses];
-  auto fetch_tile = [&](int j) __attribute__((always_inline)) {
+  // Start the asynchronous copy of KV block j into the LDS buffers kb / vb.
+  auto issue_tile = [&](int j, uint8_t* kb, uint8_t* vb) __attribute__((always_inline)) {
     const int k_base = j * kKvBlock * (int)a.k_rs, v_base = j * kKvBlock * (int)a.v_rs;
 #pragma unroll
     for (int p = 0; p < kPasses; ++p) {
-      stage_k[p] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, k_src[p], k_base, 0);
-      stage_v[p] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, v_src[p], v_base, 0);
-    }
-  };
-  auto commit_tile = [&](uint8_t* kb, uint8_t* vb) __attribute__((always_inline)) {
-#pragma unroll
-    for (int p = 0; p < kPasses; ++p) {
-      const int off = (p * 4 + wave) * 1024 + lane * 16;
-      *LDS_PTR(v4i, kb + off) = stage_k[p];
-      *LDS_PTR(v4i, vb + off) = stage_v[p];
+      const int seg = (p * 4 + wave) * 1024;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, LDS_PTR(void, kb + seg), 16, k_src[p], k_base, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(v_rsrc, LDS_PTR(void, vb + seg), 16, v_src[p], v_base, 0, 0);
     }
   };
 
@@ -272,12 +263,13 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
   float m_run = -INFINITY;  // running row max of raw S (both half-lanes of a query hold the same value)
   float l_run = 0.f;        // this lane's share of the running row sum
 
-  // The loop is software-pipelined inside every wavefront: the S^T MFMAs of block i+1 are issued before the softmax of
-  // block i and the PV MFMAs of block i right after it, so the vector ALU never waits for a matrix result that was
-  // issued just before (the matrix core runs them underneath the softmax arithmetic).
-
-  // S^T = K Q^T for the KV block held in kb: two 32(kv) x 32(q) sub-tiles.
-  auto qk_tile = [&](const uint8_t* kb, v16f (&s)[2]) __attribute__((always_inline)) {
+  // S^T, online softmax and PV for KV block j held in kb / vb.
+  auto compute_tile = [&](int j, const uint8_t* kb, const uint8_t* vb, auto masked_c) __attribute__((always_inline)) {
+    // kMasked also marks the general path (first block, diagonal, tail): only there can the running max still be -inf
+    constexpr bool kMasked = decltype(masked_c)::value;
+    const int kv0 = j * kKvBlock;
+    // ---- S^T = K Q^T : two 32(kv) x 32(q) sub-tiles ----
+    v16f s[2];
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
 #pragma unroll
@@ -290,14 +282,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
         s[t] = mfma_fp8<E5M2>(kf, qf[ks], s[t]);
       }
     }
-  };
-
-  // Online softmax of KV block j (reference softmax_rescale_o, csrc/flash_attention.cu:233-273): s -> p8, and the
-  // rescale of l and O by alpha = exp(scale * (m_old - m_new)).
-  auto softmax_tile = [&](int j, v16f (&s)[2], v8i& p8, auto masked_c) __attribute__((always_inline)) {
-    constexpr bool kMasked = decltype(masked_c)::value;
-    const int kv0 = j * kKvBlock;
-    // causal / tail mask: register i of sub-tile t is kv row kv0 + 32h + 16t + i
+    // ---- causal / tail mask: register i of sub-tile t is kv row kv0 + 32h + 16t + i ----
     const int kv_limit = CAUSAL ? min(q_row, kv_last) : kv_last;  // last kv this query attends to
     if constexpr (kMasked) {
 #pragma unroll
@@ -306,14 +291,16 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
         for (int i = 0; i < 16; ++i)
           if (kv0 + 32 * h + 16 * t + i > kv_limit) s[t][i] = -INFINITY;
     }
-    float mx[4] = {m_run, m_run, m_run, m_run};  // four independent chains
+    // ---- online softmax (reference softmax_rescale_o, csrc/flash_attention.cu:233-273) ----
+    float mx[4] = {m_run, m_run, m_run, m_run};  // four independent chains; sub-tile 0 first (it is ready first)
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int i = 0; i < 16; i += 2) mx[(i >> 1) & 3] = max3(mx[(i >> 1) & 3], s[t][i], s[t][i + 1]);
     const float m_new = lane32_max(max3(max3(mx[0], mx[1], mx[2]), mx[3], mx[3]));  // same in both half-lanes
     if (__any(m_new != m_run)) {
-      const float alpha = (m_run == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((m_run - m_new) * c);
+      float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * c);
+      if constexpr (kMasked) alpha = (m_run == -INFINITY) ? 0.f : alpha;
       l_run *= alpha;
 #pragma unroll
       for (int mt = 0; mt < kMTiles; ++mt)
@@ -321,8 +308,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
         for (int i = 0; i < 16; ++i) o_acc[mt][i] *= alpha;
       m_run = m_new;
     }
-    const float mc = (m_new == -INFINITY) ? 0.f : m_new * c;
+    float mc = m_new * c;
+    if constexpr (kMasked) mc = (m_new == -INFINITY) ? 0.f : mc;
     float sum0 = 0.f, sum1 = 0.f;
+    v8i p8;
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
 #pragma unroll
@@ -343,10 +332,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
         p8[4 * t + w] = pack4_fp8<E5M2>(s[t][4 * w], s[t][4 * w + 1], s[t][4 * w + 2], s[t][4 * w + 3]);
     }
     l_run += sum0 + sum1;
-  };
-
-  // O^T += V^T P^T for the KV block held in vb; the V^T fragment of tile mt+1 is fetched while the MFMA of mt runs.
-  auto pv_tile = [&](const uint8_t* vb, const v8i& p8) __attribute__((always_inline)) {
+    // ---- O^T += V^T P^T : the V^T fragment of tile mt+1 is fetched while the MFMA of tile mt runs ----
     auto load_vf = [&](int mt) __attribute__((always_inline)) {
       v8i vf;
 #pragma unroll
@@ -366,59 +352,55 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
       if (mt + 1 < kMTiles) vf_cur = vf_next;
     }
   };
-
-  // Three LDS stages: KV block t lives in stage t % 3.  In the step for block i the wavefront reads K of block i+1
-  // and V of block i, fetches block i+2 into registers at the start and commits it to stage (i+2) % 3 at the end
-  // (that stage held block i-1, whose V was last read in the previous step).  The barrier that ends the step makes
-  // the committed block visible and frees the stage of block i.
-  auto k_stage = [&](int t) __attribute__((always_inline)) {
-    return (t % 3) == 0 ? k_lds0 : ((t % 3) == 1 ? k_lds1 : k_lds2);
+  // Three LDS stages, copies issued two KV blocks ahead.  At the end of the step for block j the copy of block
+  // j+1 (issued one step earlier) must have landed while the copy of block j+2 (issued in this step: kLoadsPerTile
+  // loads per lane) may stay in flight; vmcnt counts this lane's loads in issue order.  The barrier then tells every
+  // wavefront that all shares of block j+1 are in LDS and that block j's stage may be overwritten.  It is a bare
+  // s_barrier: __syncthreads() would also wait for the copy that is meant to stay in flight.
+  constexpr int kLoadsPerTile = 2 * kPasses;
+  auto stage_sync = [&](bool next_in_flight) __attribute__((always_inline)) {
+    // s_waitcnt immediate (gfx9 layout): vmcnt[3:0], expcnt[6:4] = 7 and lgkmcnt[11:8] = 15 (no wait on those)
+    if (next_in_flight)
+      __builtin_amdgcn_s_waitcnt(0x0F70 | kLoadsPerTile);
+    else
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+    __builtin_amdgcn_s_barrier();
   };
-  auto v_stage = [&](int t) __attribute__((always_inline)) {
-    return (t % 3) == 0 ? v_lds0 : ((t % 3) == 1 ? v_lds1 : v_lds2);
-  };
+  static_assert(kLoadsPerTile < 16, "vmcnt immediate above");
 
-  // Prologue: blocks 0 and 1 in LDS, S of block 0 computed.
-  fetch_tile(0);
-  commit_tile(k_lds0, v_lds0);
-  if (n_tiles > 1) {
-    fetch_tile(1);
-    commit_tile(k_lds1, v_lds1);
+  issue_tile(0, k_lds0, v_lds0);
+  if (n_tiles > 1) issue_tile(1, k_lds1, v_lds1);
+  stage_sync(n_tiles > 1);
+  // Block 0 takes the general path: it is the only block that can meet a running max of -inf.
+  if (n_tiles > 2) issue_tile(2, k_lds2, v_lds2);
+  compute_tile(0, k_lds0, v_lds0, std::true_type());
+  stage_sync(n_tiles > 2);
+  int j = 1;
+  // Mask-free blocks, three per trip so that every third reads one fixed LDS stage (the compiler can then tell
+  // that the copies in flight go to other stages and need not be waited for before the reads).
+  // Inside this loop every copy is issued unconditionally (block j+4 exists), which lets the compiler see that each
+  // s_waitcnt below always leaves exactly one block in flight.
+  for (; j + 2 < n_plain && j + 4 < n_tiles; j += 3) {
+    issue_tile(j + 2, k_lds0, v_lds0);
+    compute_tile(j, k_lds1, v_lds1, std::false_type());
+    stage_sync(true);
+    issue_tile(j + 3, k_lds1, v_lds1);
+    compute_tile(j + 1, k_lds2, v_lds2, std::false_type());
+    stage_sync(true);
+    issue_tile(j + 4, k_lds2, v_lds2);
+    compute_tile(j + 2, k_lds0, v_lds0, std::false_type());
+    stage_sync(true);
   }
-  __syncthreads();
-  v16f s_a[2], s_b[2];  // S^T of the block being soft-maxed and of the next one, alternating roles
-  v8i p8;
-  qk_tile(k_lds0, s_a);
-  int j = 0;
-  // Mask-free blocks, six per trip (3 LDS stages x 2 roles of the S registers) so that every step reads fixed LDS
-  // stages and S alternates between s_a and s_b without register copies.
-#define FA8_STEP(J, S_CUR, S_NEXT, KN, VC, KW, VW)        \
-  fetch_tile((J) + 2);                                    \
-  qk_tile(KN, S_NEXT);                                    \
-  softmax_tile((J), S_CUR, p8, std::false_type());        \
-  pv_tile(VC, p8);                                        \
-  commit_tile(KW, VW);                                    \
-  __syncthreads();
-  for (; j + 5 < n_plain && j + 7 < n_tiles; j += 6) {
-    FA8_STEP(j + 0, s_a, s_b, k_lds1, v_lds0, k_lds2, v_lds2)
-    FA8_STEP(j + 1, s_b, s_a, k_lds2, v_lds1, k_lds0, v_lds0)
-    FA8_STEP(j + 2, s_a, s_b, k_lds0, v_lds2, k_lds1, v_lds1)
-    FA8_STEP(j + 3, s_b, s_a, k_lds1, v_lds0, k_lds2, v_lds2)
-    FA8_STEP(j + 4, s_a, s_b, k_lds2, v_lds1, k_lds0, v_lds0)
-    FA8_STEP(j + 5, s_b, s_a, k_lds0, v_lds2, k_lds1, v_lds1)
-  }
-#undef FA8_STEP
-  // The remaining blocks (the last few mask-free ones, the blocks on the diagonal, the kv tail) take the masking copy
-  // with run-time stage selection; S of block j is in s_a.
+  // The remaining blocks (the last few mask-free ones, the blocks on the diagonal, the kv tail) take the masking copy.
   for (; j < n_tiles; ++j) {
-    if (j + 2 < n_tiles) fetch_tile(j + 2);
-    if (j + 1 < n_tiles) qk_tile(k_stage(j + 1), s_b);
-    softmax_tile(j, s_a, p8, std::true_type());
-    pv_tile(v_stage(j), p8);
-    if (j + 2 < n_tiles) commit_tile(k_stage(j + 2), v_stage(j + 2));
-    __syncthreads();
-    s_a[0] = s_b[0];
-    s_a[1] = s_b[1];
+    const int st = j % 3, st2 = (j + 2) % 3;
+    if (j + 2 < n_tiles)
+      issue_tile(j + 2, st2 == 0 ? k_lds0 : (st2 == 1 ? k_lds1 : k_lds2), st2 == 0 ? v_lds0 : (st2 == 1 ? v_lds1 : v_lds2));
+    // a wavefront whose 32 query rows all lie before this kv block has nothing to add (causal)
+    if (!CAUSAL || j * kKvBlock <= q_wave0 + kQWave - 1)
+      compute_tile(j, st == 0 ? k_lds0 : (st == 1 ? k_lds1 : k_lds2), st == 0 ? v_lds0 : (st == 1 ? v_lds1 : v_lds2),
+                   std::true_type());
+    stage_sync(j + 2 < n_tiles);
   }
 
   // ---- epilogue: O / l, convert, store (reference csrc/flash_attention.cu:542-582) ----
