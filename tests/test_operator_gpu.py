@@ -1,0 +1,188 @@
+"""GPU tests of the operator boundary: the compiled binding `attention_cutlass_fp8`, the ctypes mirror and the raw C ABI
+must agree bit for bit; streams, determinism, guard bands, strided tensors, fp8 output, e5m2 inputs, error paths."""
+import ctypes
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import cutlass_flash_atten_fp8_amd as fa
+from oracle import fa8_oracle as fo
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def rand_fp8(shape, seed, dtype=torch.float8_e4m3fn, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype)
+
+
+def u8(t):
+    return t.view(torch.uint8).cpu().numpy()
+
+
+def abi_call(q, k, v, o, causal, scale, stream=None):
+    p = fa.make_params(q, k, v, o, causal, scale)
+    s = torch.cuda.current_stream() if stream is None else stream
+    rc = fa.lib().fa8_fwd(ctypes.byref(p), ctypes.c_void_p(s.cuda_stream))
+    assert rc == 0, fa.error_string(rc)
+    return o
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_binding_mirror_and_abi_agree_bitwise(causal):
+    ext = fa.load_extension()
+    q, k, v = (rand_fp8((2, 4, 300, 128), s).to(DEV) for s in (1, 2, 3))
+    out = ext.flash_attention_v2_cutlass(q, k, v, causal, 0.09)
+    assert isinstance(out, list) and len(out) == 1
+    o1 = out[0]
+    assert o1.dtype == torch.float16 and o1.shape == q.shape and o1.is_contiguous()
+    o2 = fa.flash_attention_v2_cutlass(q, k, v, causal, 0.09)[0]
+    o3 = abi_call(q, k, v, torch.empty_like(o1), causal, 0.09)
+    torch.cuda.synchronize()
+    assert torch.equal(o1, o2) and torch.equal(o1, o3)
+    # keyword form of the five reference arguments
+    o4 = ext.flash_attention_v2_cutlass(q=q, k=k, v=v, is_causal=causal, softmax_scale=0.09)[0]
+    assert torch.equal(o1, o4)
+
+
+def test_runs_on_the_current_stream_without_device_sync():
+    ext = fa.load_extension()
+    q, k, v = (rand_fp8((1, 8, 1024, 128), s).to(DEV) for s in (4, 5, 6))
+    ref = ext.flash_attention_v2_cutlass(q, k, v, False, 0.09)[0]
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        o = ext.flash_attention_v2_cutlass(q, k, v, False, 0.09)[0]
+        done = torch.cuda.Event()
+        done.record(side)
+    done.synchronize()
+    assert torch.equal(o, ref)
+
+
+def test_deterministic_run_to_run():
+    q, k, v = (rand_fp8((2, 8, 2000, 128), s).to(DEV) for s in (7, 8, 9))
+    outs = [fa.flash_attention_v2_cutlass(q, k, v, True, 0.09)[0] for _ in range(3)]
+    torch.cuda.synchronize()
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+
+
+@pytest.mark.parametrize("n,d", [(1, 64), (100, 64), (129, 128), (1000, 128)])
+def test_guard_bands_and_poisoned_padding(n, d):
+    """O is written only inside [B,H,N,d]; K/V bytes past row N-1 (NaN codes here) never reach the result."""
+    B, H, pad = 2, 2, 64
+    qs, ks, vs = (rand_fp8((B, H, n, d), s) for s in (10, 11, 12))
+
+    def padded(t):  # rows n..n+pad of every head are fp8 NaN (0x7F)
+        buf = torch.full((B, H, n + pad, d), 0x7F, dtype=torch.uint8)
+        buf[:, :, :n] = t.view(torch.uint8)
+        return buf.to(DEV).view(torch.float8_e4m3fn)[:, :, :n]
+
+    qp, kp, vp = padded(qs), padded(ks), padded(vs)
+    obuf = torch.full((B, H, n + pad, d), 777.0, dtype=torch.float16, device=DEV)
+    abi_call(qp, kp, vp, obuf[:, :, :n], False, 0.1)
+    o_plain = abi_call(qs.to(DEV), ks.to(DEV), vs.to(DEV), torch.empty((B, H, n, d), dtype=torch.float16, device=DEV), False, 0.1)
+    torch.cuda.synchronize()
+    assert torch.equal(obuf[:, :, :n], o_plain)
+    assert (obuf[:, :, n:] == 777.0).all()
+    assert torch.isfinite(o_plain).all()
+
+
+def test_strided_batch_and_head_layout():
+    """[B,N,H,d] storage viewed as [B,H,N,d]: arbitrary batch/head/row strides, last dim contiguous."""
+    B, H, n, d = 2, 3, 200, 128
+    qs, ks, vs = (rand_fp8((B, n, H, d), s).to(DEV) for s in (13, 14, 15))
+    q, k, v = (t.permute(0, 2, 1, 3) for t in (qs, ks, vs))
+    o = torch.empty((B, n, H, d), dtype=torch.float16, device=DEV).permute(0, 2, 1, 3)
+    abi_call(q, k, v, o, True, 0.09)
+    ref = abi_call(q.contiguous(), k.contiguous(), v.contiguous(), torch.empty((B, H, n, d), dtype=torch.float16, device=DEV), True, 0.09)
+    torch.cuda.synchronize()
+    assert torch.equal(o.contiguous(), ref)
+
+
+def test_causal_rows_do_not_see_future_keys_bitwise():
+    q, k, v = (rand_fp8((1, 4, 700, 128), s) for s in (16, 17, 18))
+    a = fa.flash_attention_v2_cutlass(q.to(DEV), k.to(DEV), v.to(DEV), True, 0.09)[0]
+    k2, v2 = k.clone(), v.clone()
+    k2[:, :, 400:] = rand_fp8((1, 4, 300, 128), 19, scale=3.0)
+    v2[:, :, 400:] = rand_fp8((1, 4, 300, 128), 20, scale=3.0)
+    b = fa.flash_attention_v2_cutlass(q.to(DEV), k2.to(DEV), v2.to(DEV), True, 0.09)[0]
+    torch.cuda.synchronize()
+    assert torch.equal(a[:, :, :400], b[:, :, :400])
+    assert not torch.equal(a[:, :, 400:], b[:, :, 400:])
+
+
+def test_closed_form_answers_on_the_gpu():
+    d, n = 128, 300
+    q, k, v = (rand_fp8((1, 2, n, d), s) for s in (21, 22, 23))
+    # causal row 0 is exactly V[0]
+    o = fa.flash_attention_v2_cutlass(q.to(DEV), k.to(DEV), v.to(DEV), True, 0.09)[0].cpu()
+    assert torch.equal(o[:, :, 0].float(), v[:, :, 0].float())
+    # scale 0: every visible weight is exactly 1 -> O = (prefix) mean of V
+    o0 = fa.flash_attention_v2_cutlass(q.to(DEV), k.to(DEV), v.to(DEV), False, 0.0)[0].float().cpu()
+    assert torch.allclose(o0, v.float().mean(dim=2, keepdim=True).expand_as(o0), atol=1e-3, rtol=0)
+    oc = fa.flash_attention_v2_cutlass(q.to(DEV), k.to(DEV), v.to(DEV), True, 0.0)[0].float().cpu()
+    prefix = torch.cumsum(v.float(), dim=2) / torch.arange(1, n + 1).view(1, 1, n, 1)
+    assert torch.allclose(oc, prefix, atol=2e-3, rtol=0)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("d", [64, 128])
+def test_fp8_output_matches_oracle(causal, d):
+    """out_dtype = e4m3: what the reference itself stores (reference csrc/flash_attention.cu:557)."""
+    q, k, v = (rand_fp8((2, 2, 260, d), s) for s in (24, 25, 26))
+    scale = 1 / math.sqrt(d)
+    o8 = fa.flash_attention_v2_cutlass(q.to(DEV), k.to(DEV), v.to(DEV), causal, scale, out_dtype=torch.float8_e4m3fn)[0]
+    o16 = fa.flash_attention_v2_cutlass(q.to(DEV), k.to(DEV), v.to(DEV), causal, scale)[0]
+    assert o8.dtype == torch.float8_e4m3fn
+    # same fp32 result rounded once to e4m3 and once to fp16: the e4m3 output must be within half an e4m3 step of the fp16 one
+    a, b = o8.float().cpu().numpy(), o16.float().cpu().numpy()
+    assert np.all(np.abs(a - b) <= np.maximum(np.abs(b) * 2.0 ** -4, 2.0 ** -10) * 1.001)
+    ref = fo.forward(u8(q), u8(k), u8(v), scale, causal=causal, exp2_form=True, out_dtype=fo.OUT_E4M3)
+    refv = torch.from_numpy(ref).view(torch.float8_e4m3fn).float().numpy()
+    err = np.abs(a - refv)
+    assert (err > 0).mean() < 0.05  # identical codes except where the fp32 value sits on a rounding boundary
+    assert err.mean() <= 2e-3
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_e5m2_inputs_match_oracle(causal):
+    q, k, v = (rand_fp8((2, 2, 333, 128), s, dtype=torch.float8_e5m2) for s in (27, 28, 29))
+    scale = 1 / math.sqrt(128)
+    o = fa.flash_attention_v2_cutlass(q.to(DEV), k.to(DEV), v.to(DEV), causal, scale)[0].float().cpu().numpy()
+    ref, allow = fo.forward(u8(q), u8(k), u8(v), scale, causal=causal, exp2_form=True, in_dtype=fo.E5M2, logit_rel_err=2e-5)
+    err = np.abs(o - ref.astype(np.float32))
+    print(f"e5m2 causal={causal}: max {err.max():.3e} mean {err.mean():.3e}")
+    assert (err.max(axis=-1) <= 2e-2 + allow).all()
+    assert err.mean() <= 2e-3
+
+
+def test_error_paths_raise_and_launch_nothing():
+    ext = fa.load_extension()
+    q = rand_fp8((1, 2, 128, 96), 30).to(DEV)
+    with pytest.raises(RuntimeError, match="head_dim"):
+        ext.flash_attention_v2_cutlass(q, q, q, False, 0.1)
+    q = rand_fp8((1, 2, 128, 128), 31).to(DEV)
+    with pytest.raises(RuntimeError, match="contiguous"):
+        ext.flash_attention_v2_cutlass(q.transpose(1, 2), q, q, False, 0.1)
+    with pytest.raises(RuntimeError, match="same dtype"):
+        ext.flash_attention_v2_cutlass(q, q.view(torch.uint8).view(torch.float8_e5m2), q, False, 0.1)
+    with pytest.raises(RuntimeError, match="float8"):
+        ext.flash_attention_v2_cutlass(q.half(), q.half(), q.half(), False, 0.1)
+    with pytest.raises(RuntimeError, match="float8"):
+        ext.flash_attention_v2_cutlass(*(t.view(torch.uint8).view(torch.float8_e4m3fnuz) for t in (q, q, q)), False, 0.1)
+    k_short = rand_fp8((1, 2, 64, 128), 32).to(DEV)
+    with pytest.raises(RuntimeError):  # causal needs seqlen_q == seqlen_k
+        ext.flash_attention_v2_cutlass(q, k_short, k_short, True, 0.1)
+    with pytest.raises(RuntimeError, match="finite"):
+        ext.flash_attention_v2_cutlass(q, q, q, False, float("nan"))
+    with pytest.raises(RuntimeError):  # the [B,H,d,N] layout is validated but has no kernel yet
+        ext.flash_attention_v2_cutlass(q, q, q.transpose(2, 3).contiguous(), False, 0.1, v_transposed=True)
+    torch.cuda.synchronize()
+    # seqlen_q != seqlen_k is fine without the causal mask
+    o = ext.flash_attention_v2_cutlass(q, k_short, k_short, False, 0.1)[0]
+    ref = fo.forward(u8(q), u8(k_short), u8(k_short), 0.1, exp2_form=True).astype(np.float32)
+    assert np.abs(o.float().cpu().numpy() - ref).mean() <= 2e-3
