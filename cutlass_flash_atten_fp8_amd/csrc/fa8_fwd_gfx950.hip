@@ -154,7 +154,7 @@ __device__ __forceinline__ void decode_block(const KernelArgs& a, int id, int& b
   qb = CAUSAL ? (a.n_qblocks - 1 - qi) : qi;
 }
 
-template <int D, bool CAUSAL, bool E5M2, int OUT>
+template <int D, bool CAUSAL, bool E5M2, int OUT, bool VT>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WAVES_PER_EU))) void fa8_fwd_kernel(
     const KernelArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the body uses device-only types (buffer resources); the host pass only needs the stub
@@ -211,23 +211,40 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
     int r, ch;
     tile_slot_decode<D, false>(slot, r, ch);
     k_src[p] = (unsigned)(kv_of_lds_row(r) * (int)a.k_rs + ch * 16);
-    tile_slot_decode<D, true>(slot, r, ch);
-    v_src[p] = (unsigned)(r * (int)a.v_rs + ch * 16);
+    if constexpr (VT) {
+      // v is [d, Nk]: the tile is D rows of 64 kv bytes (4 chunks), laid out like a 64-byte-row K tile
+      tile_slot_decode<64, false>(slot, r, ch);
+      v_src[p] = (unsigned)(r * (int)a.v_rs + ch * 16);
+    } else {
+      tile_slot_decode<D, true>(slot, r, ch);
+      v_src[p] = (unsigned)(r * (int)a.v_rs + ch * 16);
+    }
   }
   const int kv_last = a.seqlen_k - 1;
   constexpr int kRsrcFlags = 0x00020000;  // raw buffer, 32-bit data format
   const __amdgpu_buffer_rsrc_t k_rsrc =
       __builtin_amdgcn_make_buffer_rsrc((void*)kp, 0, (int)(kv_last * a.k_rs + D), kRsrcFlags);
-  const __amdgpu_buffer_rsrc_t v_rsrc =
-      __builtin_amdgcn_make_buffer_rsrc((void*)vp, 0, (int)(kv_last * a.v_rs + D), kRsrcFlags);
+  const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)vp, 0, VT ? (int)((D - 1) * a.v_rs + a.seqlen_k) : (int)(kv_last * a.v_rs + D), kRsrcFlags);
   // Start the asynchronous copy of KV block j into the LDS buffers kb / vb.
   auto issue_tile = [&](int j, uint8_t* kb, uint8_t* vb) __attribute__((always_inline)) {
-    const int k_base = j * kKvBlock * (int)a.k_rs, v_base = j * kKvBlock * (int)a.v_rs;
+    const int k_base = j * kKvBlock * (int)a.k_rs;
+    const int v_base = VT ? j * kKvBlock : j * kKvBlock * (int)a.v_rs;
+    // transposed v, ragged last block: the 16-byte chunks past the last kv column would read the start of the next
+    // head-dim row (or run off the tensor); they are pulled back onto the last chunk instead (and masked later)
+    const bool v_clamp = VT && (j + 1) * kKvBlock > a.seqlen_k;
 #pragma unroll
     for (int p = 0; p < kPasses; ++p) {
       const int seg = (p * 4 + wave) * 1024;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, LDS_PTR(void, kb + seg), 16, k_src[p], k_base, 0, 0);
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(v_rsrc, LDS_PTR(void, vb + seg), 16, v_src[p], v_base, 0, 0);
+      if (v_clamp) {
+        int r, ch;
+        tile_slot_decode<64, false>((p * 4 + wave) * 64 + lane, r, ch);
+        const unsigned off = (unsigned)(r * (int)a.v_rs + min(v_base + ch * 16, a.seqlen_k - 16));
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(v_rsrc, LDS_PTR(void, vb + seg), 16, off, 0, 0, 0);
+      } else {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(v_rsrc, LDS_PTR(void, vb + seg), 16, v_src[p], v_base, 0, 0);
+      }
     }
   };
 
@@ -244,9 +261,13 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
   // 2j and 2j+1 address the two 8-byte halves of kv row j of an 8 x 16 byte block, and lane i receives
   // byte i of each of the 8 rows: 8 consecutive kv for one head-dim column.
   const int tr_j = (lane & 15) >> 1, tr_e = lane & 1, tr_g1 = (lane >> 4) & 1;
-  int v_off[kMTiles];
+  // (transposed v: the tile already is V^T, [d][64 kv]: plain 16-byte reads of row 32mt + lane % 32, chunks 2h, 2h+1)
+  int v_off[kMTiles], vt_off[2];
 #pragma unroll
   for (int mt = 0; mt < kMTiles; ++mt) v_off[mt] = tile_offset<D, true>(32 * h + tr_j, 2 * mt + tr_g1) + 8 * tr_e;
+#pragma unroll
+  for (int e = 0; e < 2; ++e) vt_off[e] = tile_offset<64, false>(qn, 2 * h + e);
+  constexpr int kVtTileStride = 32 * 64;  // LDS bytes between 32-row groups of the [d][64] tile
   constexpr int kTrStride = 8 * D;  // LDS bytes between successive groups of 8 kv rows
 
   const int n_tiles = CAUSAL ? (min(a.seqlen_k, q0 + kQBlock) + kKvBlock - 1) / kKvBlock
@@ -335,11 +356,17 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
     // ---- O^T += V^T P^T : the V^T fragment of tile mt+1 is fetched while the MFMA of tile mt runs ----
     auto load_vf = [&](int mt) __attribute__((always_inline)) {
       v8i vf;
+      if constexpr (VT) {
+        const v4i lo = *LDS_PTR(const v4i, vb + mt * kVtTileStride + vt_off[0]);
+        const v4i hi = *LDS_PTR(const v4i, vb + mt * kVtTileStride + vt_off[1]);
+        vf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      } else {
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const v2i r = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_PTR(v2i, vb + v_off[mt] + g * kTrStride));
-        vf[2 * g] = r[0];
-        vf[2 * g + 1] = r[1];
+        for (int g = 0; g < 4; ++g) {
+          const v2i r = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_PTR(v2i, vb + v_off[mt] + g * kTrStride));
+          vf[2 * g] = r[0];
+          vf[2 * g + 1] = r[1];
+        }
       }
       return vf;
     };
@@ -439,20 +466,23 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
 }
 
 template <int D, bool CAUSAL, bool E5M2, int OUT>
-int launch(const KernelArgs& a, hipStream_t stream) {
+int launch(const KernelArgs& a, bool v_transposed, hipStream_t stream) {
   const dim3 grid((unsigned)(a.bh_total * a.n_qblocks));
-  hipLaunchKernelGGL((fa8_fwd_kernel<D, CAUSAL, E5M2, OUT>), grid, dim3(kThreads), 0, stream, a);
+  if (v_transposed)
+    hipLaunchKernelGGL((fa8_fwd_kernel<D, CAUSAL, E5M2, OUT, true>), grid, dim3(kThreads), 0, stream, a);
+  else
+    hipLaunchKernelGGL((fa8_fwd_kernel<D, CAUSAL, E5M2, OUT, false>), grid, dim3(kThreads), 0, stream, a);
   return (int)hipGetLastError();
 }
 
 template <int D, bool CAUSAL>
 int launch_types(const Fa8FwdParams* p, const KernelArgs& a, hipStream_t stream) {
-  const bool e5m2 = p->in_dtype == FA8_DTYPE_E5M2;
+  const bool e5m2 = p->in_dtype == FA8_DTYPE_E5M2, vt = p->v_layout == FA8_V_TRANSPOSED;
   if (p->out_dtype == FA8_OUT_FP16)
-    return e5m2 ? launch<D, CAUSAL, true, FA8_OUT_FP16>(a, stream) : launch<D, CAUSAL, false, FA8_OUT_FP16>(a, stream);
+    return e5m2 ? launch<D, CAUSAL, true, FA8_OUT_FP16>(a, vt, stream) : launch<D, CAUSAL, false, FA8_OUT_FP16>(a, vt, stream);
   // fp8 output: the reference stores O in the input element type; only e4m3 out of e4m3 in is built
   if (e5m2) return FA8_ERR_UNSUPPORTED;
-  return launch<D, CAUSAL, false, FA8_OUT_E4M3>(a, stream);
+  return launch<D, CAUSAL, false, FA8_OUT_E4M3>(a, vt, stream);
 }
 
 bool span_ok(long long outer_stride, long long inner_extent) { return outer_stride >= inner_extent; }
@@ -490,7 +520,8 @@ extern "C" int fa8_fwd_validate(const Fa8FwdParams* p) {
   if ((uintptr_t)p->o % 8 != 0) return FA8_ERR_ALIGN;
   // the kernels address k and v of one head with 32-bit byte offsets
   if ((long long)p->seqlen_k * p->k_row_stride > 0x7fffffffLL || v_rows * p->v_row_stride > 0x7fffffffLL) return FA8_ERR_SHAPE;
-  if (p->v_layout == FA8_V_TRANSPOSED) return FA8_ERR_UNSUPPORTED;
+  // transposed v is read in 16-byte chunks along kv
+  if (p->v_layout == FA8_V_TRANSPOSED && p->seqlen_k % 16 != 0) return FA8_ERR_ALIGN;
   if (p->in_dtype == FA8_DTYPE_E5M2 && p->out_dtype == FA8_OUT_E4M3) return FA8_ERR_UNSUPPORTED;
   return FA8_OK;
 }

@@ -39,7 +39,7 @@ extern "C" {
 #define FA8_ERR_SHAPE (-2)       /* a size is < 1, or causal with seqlen_q != seqlen_k */
 #define FA8_ERR_HEAD_DIM (-3)    /* head_dim is not one of the compiled buckets (64, 128) */
 #define FA8_ERR_STRIDE (-4)      /* a stride is smaller than the extent it must span, or rows overlap */
-#define FA8_ERR_ALIGN (-5)       /* a base pointer or stride breaks the 16-byte row alignment the kernels load with */
+#define FA8_ERR_ALIGN (-5)       /* a base pointer or stride breaks the 16-byte row alignment the kernels load with (FA8_V_TRANSPOSED: also seqlen_k % 16 != 0) */
 #define FA8_ERR_DTYPE (-6)       /* unknown in_dtype/out_dtype/v_layout code */
 #define FA8_ERR_UNSUPPORTED (-7) /* a valid combination that this build has no kernel for */
 #define FA8_ERR_SCALE (-8)       /* softmax_scale is NaN or infinite */

@@ -84,6 +84,11 @@ def test_validate_rejects_bad_arguments():
     assert validate(p) == -6
     p = fa.make_params(q, k, v, o, False, 0.125); p.out_dtype = 9
     assert validate(p) == -6
+    vt = torch.zeros((1, 2, 64, 72), dtype=torch.float32).to(torch.float8_e4m3fn)[..., :64]  # [B,H,d,N], row stride 72
+    p = fa.make_params(q, k, vt, o, False, 0.125, v_transposed=True)
+    assert validate(p) == -5
+    vt = torch.zeros((1, 2, 64, 64), dtype=torch.float32).to(torch.float8_e4m3fn)
+    assert validate(fa.make_params(q, k, vt, o, False, 0.125, v_transposed=True)) == 0
     for bad in (float("nan"), float("inf")):
         assert validate(fa.make_params(q, k, v, o, False, bad)) == -8
 

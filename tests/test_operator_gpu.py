@@ -160,6 +160,22 @@ def test_e5m2_inputs_match_oracle(causal):
     assert err.mean() <= 2e-3
 
 
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("n,d", [(64, 64), (208, 64), (256, 128), (1008, 128)])
+def test_transposed_v_is_the_reference_calling_convention(n, d, causal):
+    """v_transposed=True takes v as [B,H,d,N], what the reference requires of its caller (reference test.py:71);
+    the result is bit-identical to the [B,H,N,d] call."""
+    ext = fa.load_extension()
+    q, k, v = (rand_fp8((2, 3, n, d), s).to(DEV) for s in (40, 41, 42))
+    o = ext.flash_attention_v2_cutlass(q, k, v, causal, 0.1)[0]
+    vt = v.transpose(2, 3).contiguous()
+    ot = ext.flash_attention_v2_cutlass(q, k, vt, causal, 0.1, v_transposed=True)[0]
+    torch.cuda.synchronize()
+    assert torch.equal(o, ot)
+    ref = fo.forward(u8(q.cpu()), u8(k.cpu()), u8(vt.cpu()), 0.1, causal=causal, exp2_form=True, v_transposed=True)
+    assert np.abs(ot.float().cpu().numpy() - ref.astype(np.float32)).mean() <= 2e-3
+
+
 def test_error_paths_raise_and_launch_nothing():
     ext = fa.load_extension()
     q = rand_fp8((1, 2, 128, 96), 30).to(DEV)
@@ -179,8 +195,9 @@ def test_error_paths_raise_and_launch_nothing():
         ext.flash_attention_v2_cutlass(q, k_short, k_short, True, 0.1)
     with pytest.raises(RuntimeError, match="finite"):
         ext.flash_attention_v2_cutlass(q, q, q, False, float("nan"))
-    with pytest.raises(RuntimeError):  # the [B,H,d,N] layout is validated but has no kernel yet
-        ext.flash_attention_v2_cutlass(q, q, q.transpose(2, 3).contiguous(), False, 0.1, v_transposed=True)
+    q100 = rand_fp8((1, 2, 100, 128), 33).to(DEV)
+    with pytest.raises(RuntimeError, match="aligned"):  # the [B,H,d,N] layout is read in 16-byte chunks along N
+        ext.flash_attention_v2_cutlass(q100, q100, q100.transpose(2, 3).contiguous(), False, 0.1, v_transposed=True)
     torch.cuda.synchronize()
     # seqlen_q != seqlen_k is fine without the causal mask
     o = ext.flash_attention_v2_cutlass(q, k_short, k_short, False, 0.1)[0]
