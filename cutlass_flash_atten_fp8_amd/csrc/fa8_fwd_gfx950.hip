@@ -1,7 +1,8 @@
 // FP8 flash-attention forward for gfx950 (MI355X): kernels and the C-ABI launcher (libfa8.so).
 //
 // One workgroup = 4 wavefronts = 128 query rows of one (batch, head); every wavefront owns 32 query
-// rows and the whole head dimension.  KV is walked in ascending blocks of 64 rows, the block size
+// rows and the whole head dimension (a multiple of 32 up to 256: the bucket sizes of the reference's
+// dispatch, csrc/static_switch.h:50-77).  KV is walked in ascending blocks of 64 rows, the block size
 // the reference instantiates (kBlockM = kBlockN = 64, reference csrc/flash_attention.cu:624), so the
 // running max that P is quantised against evolves exactly as in the reference loop
 // (csrc/flash_attention.cu:468-534).
@@ -17,8 +18,8 @@
 //     (kv_of_lds_row below); this replaces the reference's accumulator-to-A-operand reshuffle
 //     (csrc/reg2reg.h:31-96).  V^T fragments come from the row-major V tile in LDS through the
 //     transposing LDS read ds_read_b64_tr_b8, so V is consumed as [B,H,N,d] with no extra pass.
-//   * K and V tiles go HBM -> LDS with global_load_lds_dwordx4 (no register staging), double
-//     buffered, one barrier per KV block; 16-byte chunks are XOR-swizzled against bank conflicts,
+//   * K and V tiles go HBM -> LDS with buffer_load_dwordx4 ... lds (no register staging), two or three
+//     stages, one barrier per KV block; 16-byte chunks are XOR-swizzled against bank conflicts,
 //     the swizzle being applied on the global-address side of the copy.
 #include <hip/hip_runtime.h>
 
@@ -28,9 +29,9 @@
 
 #include "fa8_api.h"
 
-#ifndef FA8_WAVES_PER_EU
-#define FA8_WAVES_PER_EU 3  // at most 168 VGPRs per lane
-#endif
+// wavefronts per SIMD the kernels are compiled for: 3 (at most 168 VGPRs per lane) up to head dim 128, 2 (256 VGPRs:
+// the output accumulators alone take 128) for head dim 256
+#define FA8_WAVES_PER_EU(D) ((D) > 128 ? 2 : 3)
 
 namespace {
 
@@ -70,32 +71,49 @@ __device__ __forceinline__ int kv_of_lds_row(int r) {
   return 32 * h + 16 * t + 4 * a + b;
 }
 
-// Swizzle: a tile is an array of 128-byte lines of eight 16-byte chunks.  For D = 128 a line is a
-// row; for D = 64 a line is two rows.  chunk_slot() gives the chunk position inside the line.
+// Swizzle: a tile is an array of 128-byte lines of eight 16-byte chunks.  A row of D bytes is two lines (D = 256),
+// one line (128), half a line (64) or a quarter (32).  The chunk position inside its line is XORed with a key
+// taken from the row (line) number, chosen so that the eight lanes the LDS serves together (eight consecutive
+// rows, same chunk) fall on eight different positions, for the K reads and for the transposing V reads alike.
 template <int D, bool IS_V>
 __device__ __forceinline__ int tile_offset(int row, int chunk) {
-  if constexpr (D == 128) {
+  if constexpr (D == 256) {
+    const int key = IS_V ? (row & 7) : ((row & 7) ^ ((row >> 3) & 1));
+    return row * 256 + ((chunk >> 3) << 7) + (((chunk & 7) ^ key) << 4);
+  } else if constexpr (D == 128) {
     const int key = IS_V ? (row & 7) : ((row & 7) ^ ((row >> 3) & 1));
     return row * 128 + ((chunk ^ key) << 4);
-  } else {
+  } else if constexpr (D == 64) {
     const int line = row >> 1;
     const int key = IS_V ? (line & 3) : ((line & 3) ^ ((line >> 2) & 1));
     return line * 128 + ((((row & 1) << 2) | (chunk ^ key)) << 4);
+  } else {
+    static_assert(D == 32, "head dims: 32, 64, 128, 256");
+    const int line = row >> 2;
+    return line * 128 + ((((row & 3) << 1) | (chunk ^ (line & 1))) << 4);
   }
 }
 
 // Inverse of tile_offset for the copy engine: which (row, chunk) lives at 16-byte slot `slot`.
 template <int D, bool IS_V>
 __device__ __forceinline__ void tile_slot_decode(int slot, int& row, int& chunk) {
-  if constexpr (D == 128) {
+  if constexpr (D == 256) {
+    row = slot >> 4;
+    const int key = IS_V ? (row & 7) : ((row & 7) ^ ((row >> 3) & 1));
+    chunk = (slot & 8) | ((slot & 7) ^ key);
+  } else if constexpr (D == 128) {
     row = slot >> 3;
     const int key = IS_V ? (row & 7) : ((row & 7) ^ ((row >> 3) & 1));
     chunk = (slot & 7) ^ key;
-  } else {
+  } else if constexpr (D == 64) {
     const int line = slot >> 3, w = slot & 7;
     const int key = IS_V ? (line & 3) : ((line & 3) ^ ((line >> 2) & 1));
     row = line * 2 + (w >> 2);
     chunk = (w & 3) ^ key;
+  } else {
+    const int line = slot >> 3, w = slot & 7;
+    row = line * 4 + (w >> 1);
+    chunk = (w & 1) ^ (line & 1);
   }
 }
 
@@ -155,21 +173,30 @@ __device__ __forceinline__ void decode_block(const KernelArgs& a, int id, int& b
 }
 
 template <int D, bool CAUSAL, bool E5M2, int OUT, bool VT>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WAVES_PER_EU))) void fa8_fwd_kernel(
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WAVES_PER_EU(D)))) void fa8_fwd_kernel(
     const KernelArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the body uses device-only types (buffer resources); the host pass only needs the stub
-  constexpr int kTileBytes = kKvBlock * D;      // one K or V tile
-  constexpr int kPasses = kTileBytes / (kThreads * 16);
-  constexpr int kKSteps = D / 64;  // MFMA k-steps over the head dim for S^T
-  constexpr int kMTiles = D / 32;  // 32-row tiles of O^T
+  static_assert(D % 32 == 0 && D >= 32 && D <= 256, "head dims: multiples of 32 up to 256");
+  // LDS tiles are laid out for the next power of two: rows of DP bytes, of which the first D are used
+  constexpr int DP = D <= 32 ? 32 : (D <= 64 ? 64 : (D <= 128 ? 128 : 256));
+  constexpr int kTileBytes = kKvBlock * DP;  // one K or V tile
+  // copy passes per tile: one pass is 256 lanes x 16 bytes.  A 32-wide tile is half a pass: there wavefronts 0-1 copy
+  // K and wavefronts 2-3 copy V in one common pass.
+  constexpr bool kSplitPass = kTileBytes < kThreads * 16;
+  constexpr int kPasses = kSplitPass ? 1 : kTileBytes / (kThreads * 16);
+  constexpr int kKSteps = (D + 63) / 64;  // MFMA k-steps over the head dim for S^T (D % 64 == 32: the last one is half zeros)
+  constexpr int kMTiles = D / 32;         // 32-row tiles of O^T
+  // LDS stages per operand: three (copies issued two KV blocks ahead) where three workgroups then still fit in the
+  // 160 KB of a CU, two for head dims above 128 (2 x 32 KB per workgroup, two workgroups per CU)
+  constexpr int kStages = D > 128 ? 2 : 3;
   // One LDS object per (stage, operand): the compiler then knows that the asynchronous HBM -> LDS copy into one
   // stage cannot alias the reads of the other stage and does not wait for the copy before those reads.
   __shared__ __attribute__((aligned(1024))) uint8_t k_lds0[kTileBytes];
   __shared__ __attribute__((aligned(1024))) uint8_t k_lds1[kTileBytes];
-  __shared__ __attribute__((aligned(1024))) uint8_t k_lds2[kTileBytes];
+  __shared__ __attribute__((aligned(1024))) uint8_t k_lds2[kStages == 3 ? kTileBytes : 16];
   __shared__ __attribute__((aligned(1024))) uint8_t v_lds0[kTileBytes];
   __shared__ __attribute__((aligned(1024))) uint8_t v_lds1[kTileBytes];
-  __shared__ __attribute__((aligned(1024))) uint8_t v_lds2[kTileBytes];
+  __shared__ __attribute__((aligned(1024))) uint8_t v_lds2[kStages == 3 ? kTileBytes : 16];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keep it (and all it feeds) in scalar registers
@@ -187,37 +214,45 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
   const float c = a.scale_log2;
 
   // ---- Q fragment (B operand of S^T = K Q^T): row q_row, bytes [64ks + 32h, +32) ----
+  // (D % 64 == 32: the upper half of the last k-step does not exist; those lanes hold zeros and load nothing)
   v8i qf[kKSteps];
   {
     const int qr = min(q_row, a.seqlen_q - 1);
-    const uint8_t* src = qp + (long long)qr * a.q_rs + 32 * h;
+    const uint8_t* src = qp + (long long)qr * a.q_rs;
 #pragma unroll
     for (int ks = 0; ks < kKSteps; ++ks) {
-      const v4i lo = *(const v4i*)(src + 64 * ks);
-      const v4i hi = *(const v4i*)(src + 64 * ks + 16);
+      const bool upper_exists = 64 * ks + 32 < D;
+      const uint8_t* s8 = src + 64 * ks + (upper_exists ? 32 * h : 0);
+      const v4i lo = *(const v4i*)(s8);
+      const v4i hi = *(const v4i*)(s8 + 16);
       qf[ks] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      if (!upper_exists && h) qf[ks] = v8i{0, 0, 0, 0, 0, 0, 0, 0};
     }
   }
 
   // ---- HBM -> LDS copy: buffer_load_dwordx4 ... lds ----
   // In pass p wavefront w fills LDS bytes [(4p+w)*1024, +1024) of the tile, lane l the 16 bytes at +16l; which
-  // (kv row, 16-byte chunk) belongs there follows from the swizzle.  The source address is the head's base (buffer
-  // resource) + a per-lane byte offset that never changes (VGPR) + the block's byte offset (SGPR): no vector ALU
-  // work per block.  The resource ends with the last kv row, so rows past the end of a ragged last block read 0.
+  // (kv row, 16-byte chunk) belongs there follows from the swizzle.  (A 32-wide tile is 2 KB: wavefronts 0-1 fill the K
+  // tile, wavefronts 2-3 the V tile.)  The source address is the head's base (buffer resource) + a per-lane byte
+  // offset that never changes (VGPR) + the block's byte offset (SGPR): no vector ALU work per block.  The resource
+  // ends with the last kv row, so rows past the end of a ragged last block read 0.  LDS chunks that lie past the
+  // head dim (D < DP) get an offset beyond any resource and read 0 as well: the K fragments of a half k-step rely on it.
+  constexpr unsigned kNoSource = 0x80000000u;
+  auto copy_segment = [&](int p) __attribute__((always_inline)) { return kSplitPass ? (wave & 1) : (p * 4 + wave); };
   unsigned k_src[kPasses], v_src[kPasses];
 #pragma unroll
   for (int p = 0; p < kPasses; ++p) {
-    const int slot = (p * 4 + wave) * 64 + lane;
+    const int slot = copy_segment(p) * 64 + lane;
     int r, ch;
-    tile_slot_decode<D, false>(slot, r, ch);
-    k_src[p] = (unsigned)(kv_of_lds_row(r) * (int)a.k_rs + ch * 16);
+    tile_slot_decode<DP, false>(slot, r, ch);
+    k_src[p] = ch * 16 < D ? (unsigned)(kv_of_lds_row(r) * (int)a.k_rs + ch * 16) : kNoSource;
     if constexpr (VT) {
       // v is [d, Nk]: the tile is D rows of 64 kv bytes (4 chunks), laid out like a 64-byte-row K tile
       tile_slot_decode<64, false>(slot, r, ch);
-      v_src[p] = (unsigned)(r * (int)a.v_rs + ch * 16);
+      v_src[p] = r < D ? (unsigned)(r * (int)a.v_rs + ch * 16) : kNoSource;
     } else {
-      tile_slot_decode<D, true>(slot, r, ch);
-      v_src[p] = (unsigned)(r * (int)a.v_rs + ch * 16);
+      tile_slot_decode<DP, true>(slot, r, ch);
+      v_src[p] = ch * 16 < D ? (unsigned)(r * (int)a.v_rs + ch * 16) : kNoSource;
     }
   }
   const int kv_last = a.seqlen_k - 1;
@@ -235,28 +270,33 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
     const bool v_clamp = VT && (j + 1) * kKvBlock > a.seqlen_k;
 #pragma unroll
     for (int p = 0; p < kPasses; ++p) {
-      const int seg = (p * 4 + wave) * 1024;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, LDS_PTR(void, kb + seg), 16, k_src[p], k_base, 0, 0);
-      if (v_clamp) {
-        int r, ch;
-        tile_slot_decode<64, false>((p * 4 + wave) * 64 + lane, r, ch);
-        const unsigned off = (unsigned)(r * (int)a.v_rs + min(v_base + ch * 16, a.seqlen_k - 16));
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(v_rsrc, LDS_PTR(void, vb + seg), 16, off, 0, 0, 0);
-      } else {
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(v_rsrc, LDS_PTR(void, vb + seg), 16, v_src[p], v_base, 0, 0);
+      const int seg = copy_segment(p) * 1024;
+      if (!kSplitPass || wave < 2)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, LDS_PTR(void, kb + seg), 16, k_src[p], k_base, 0, 0);
+      if (!kSplitPass || wave >= 2) {
+        if (v_clamp) {
+          int r, ch;
+          tile_slot_decode<64, false>(copy_segment(p) * 64 + lane, r, ch);
+          const unsigned off = r < D ? (unsigned)(r * (int)a.v_rs + min(v_base + ch * 16, a.seqlen_k - 16)) : kNoSource;
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(v_rsrc, LDS_PTR(void, vb + seg), 16, off, 0, 0, 0);
+        } else {
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(v_rsrc, LDS_PTR(void, vb + seg), 16, v_src[p], v_base, 0, 0);
+        }
       }
     }
   };
 
   // ---- per-lane LDS read offsets ----
   // K fragment (A operand of S^T): the lane's row inside the 32-row MFMA tile is lane % 32 and its k-group
-  // lane / 32: chunks 4ks+2h and 4ks+2h+1 of LDS row 32t + lane % 32.
+  // lane / 32: chunks 4ks+2h and 4ks+2h+1 of LDS row 32t + lane % 32.  (Head dim 32: both k-groups read chunks 0
+  // and 1; the upper group meets the zeros of the Q fragment.  Head dims 96, 160, 224: the upper group of the last
+  // k-step reads zero-filled chunks.)
   int k_off[kKSteps][2];
 #pragma unroll
   for (int ks = 0; ks < kKSteps; ++ks)
 #pragma unroll
-    for (int e = 0; e < 2; ++e) k_off[ks][e] = tile_offset<D, false>(qn, 4 * ks + 2 * h + e);
-  constexpr int kSubTileStride = 32 * D;  // LDS bytes between S^T sub-tiles (32 rows)
+    for (int e = 0; e < 2; ++e) k_off[ks][e] = tile_offset<DP, false>(qn, DP >= 64 ? 4 * ks + 2 * h + e : e);
+  constexpr int kSubTileStride = 32 * DP;  // LDS bytes between S^T sub-tiles (32 rows)
   // V^T fragment (A operand of O^T = V^T P^T) through ds_read_b64_tr_b8: inside a group of 16 lanes, lanes
   // 2j and 2j+1 address the two 8-byte halves of kv row j of an 8 x 16 byte block, and lane i receives
   // byte i of each of the 8 rows: 8 consecutive kv for one head-dim column.
@@ -264,11 +304,11 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
   // (transposed v: the tile already is V^T, [d][64 kv]: plain 16-byte reads of row 32mt + lane % 32, chunks 2h, 2h+1)
   int v_off[kMTiles], vt_off[2];
 #pragma unroll
-  for (int mt = 0; mt < kMTiles; ++mt) v_off[mt] = tile_offset<D, true>(32 * h + tr_j, 2 * mt + tr_g1) + 8 * tr_e;
+  for (int mt = 0; mt < kMTiles; ++mt) v_off[mt] = tile_offset<DP, true>(32 * h + tr_j, 2 * mt + tr_g1) + 8 * tr_e;
 #pragma unroll
   for (int e = 0; e < 2; ++e) vt_off[e] = tile_offset<64, false>(qn, 2 * h + e);
   constexpr int kVtTileStride = 32 * 64;  // LDS bytes between 32-row groups of the [d][64] tile
-  constexpr int kTrStride = 8 * D;  // LDS bytes between successive groups of 8 kv rows
+  constexpr int kTrStride = 8 * DP;  // LDS bytes between successive groups of 8 kv rows
 
   const int n_tiles = CAUSAL ? (min(a.seqlen_k, q0 + kQBlock) + kKvBlock - 1) / kKvBlock
                              : (a.seqlen_k + kKvBlock - 1) / kKvBlock;
@@ -379,12 +419,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
       if (mt + 1 < kMTiles) vf_cur = vf_next;
     }
   };
-  // Three LDS stages, copies issued two KV blocks ahead.  At the end of the step for block j the copy of block
+  // Three LDS stages: copies issued two KV blocks ahead.  At the end of the step for block j the copy of block
   // j+1 (issued one step earlier) must have landed while the copy of block j+2 (issued in this step: kLoadsPerTile
   // loads per lane) may stay in flight; vmcnt counts this lane's loads in issue order.  The barrier then tells every
   // wavefront that all shares of block j+1 are in LDS and that block j's stage may be overwritten.  It is a bare
   // s_barrier: __syncthreads() would also wait for the copy that is meant to stay in flight.
-  constexpr int kLoadsPerTile = 2 * kPasses;
+  constexpr int kLoadsPerTile = kSplitPass ? 1 : 2 * kPasses;
   auto stage_sync = [&](bool next_in_flight) __attribute__((always_inline)) {
     // s_waitcnt immediate (gfx9 layout): vmcnt[3:0], expcnt[6:4] = 7 and lgkmcnt[11:8] = 15 (no wait on those)
     if (next_in_flight)
@@ -395,39 +435,64 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
   };
   static_assert(kLoadsPerTile < 16, "vmcnt immediate above");
 
-  issue_tile(0, k_lds0, v_lds0);
-  if (n_tiles > 1) issue_tile(1, k_lds1, v_lds1);
-  stage_sync(n_tiles > 1);
-  // Block 0 takes the general path: it is the only block that can meet a running max of -inf.
-  if (n_tiles > 2) issue_tile(2, k_lds2, v_lds2);
-  compute_tile(0, k_lds0, v_lds0, std::true_type());
-  stage_sync(n_tiles > 2);
-  int j = 1;
-  // Mask-free blocks, three per trip so that every third reads one fixed LDS stage (the compiler can then tell
-  // that the copies in flight go to other stages and need not be waited for before the reads).
-  // Inside this loop every copy is issued unconditionally (block j+4 exists), which lets the compiler see that each
-  // s_waitcnt below always leaves exactly one block in flight.
-  for (; j + 2 < n_plain && j + 4 < n_tiles; j += 3) {
-    issue_tile(j + 2, k_lds0, v_lds0);
-    compute_tile(j, k_lds1, v_lds1, std::false_type());
-    stage_sync(true);
-    issue_tile(j + 3, k_lds1, v_lds1);
-    compute_tile(j + 1, k_lds2, v_lds2, std::false_type());
-    stage_sync(true);
-    issue_tile(j + 4, k_lds2, v_lds2);
-    compute_tile(j + 2, k_lds0, v_lds0, std::false_type());
-    stage_sync(true);
-  }
-  // The remaining blocks (the last few mask-free ones, the blocks on the diagonal, the kv tail) take the masking copy.
-  for (; j < n_tiles; ++j) {
-    const int st = j % 3, st2 = (j + 2) % 3;
-    if (j + 2 < n_tiles)
-      issue_tile(j + 2, st2 == 0 ? k_lds0 : (st2 == 1 ? k_lds1 : k_lds2), st2 == 0 ? v_lds0 : (st2 == 1 ? v_lds1 : v_lds2));
-    // a wavefront whose 32 query rows all lie before this kv block has nothing to add (causal)
-    if (!CAUSAL || j * kKvBlock <= q_wave0 + kQWave - 1)
-      compute_tile(j, st == 0 ? k_lds0 : (st == 1 ? k_lds1 : k_lds2), st == 0 ? v_lds0 : (st == 1 ? v_lds1 : v_lds2),
-                   std::true_type());
-    stage_sync(j + 2 < n_tiles);
+  if constexpr (kStages == 3) {
+    issue_tile(0, k_lds0, v_lds0);
+    if (n_tiles > 1) issue_tile(1, k_lds1, v_lds1);
+    stage_sync(n_tiles > 1);
+    // Block 0 takes the general path: it is the only block that can meet a running max of -inf.
+    if (n_tiles > 2) issue_tile(2, k_lds2, v_lds2);
+    compute_tile(0, k_lds0, v_lds0, std::true_type());
+    stage_sync(n_tiles > 2);
+    int j = 1;
+    // Mask-free blocks, three per trip so that every third reads one fixed LDS stage (the compiler can then tell
+    // that the copies in flight go to other stages and need not be waited for before the reads).
+    // Inside this loop every copy is issued unconditionally (block j+4 exists), which lets the compiler see that each
+    // s_waitcnt below always leaves exactly one block in flight.
+    for (; j + 2 < n_plain && j + 4 < n_tiles; j += 3) {
+      issue_tile(j + 2, k_lds0, v_lds0);
+      compute_tile(j, k_lds1, v_lds1, std::false_type());
+      stage_sync(true);
+      issue_tile(j + 3, k_lds1, v_lds1);
+      compute_tile(j + 1, k_lds2, v_lds2, std::false_type());
+      stage_sync(true);
+      issue_tile(j + 4, k_lds2, v_lds2);
+      compute_tile(j + 2, k_lds0, v_lds0, std::false_type());
+      stage_sync(true);
+    }
+    // The remaining blocks (the last few mask-free ones, the blocks on the diagonal, the kv tail) take the masking copy.
+    for (; j < n_tiles; ++j) {
+      const int st = j % 3, st2 = (j + 2) % 3;
+      if (j + 2 < n_tiles)
+        issue_tile(j + 2, st2 == 0 ? k_lds0 : (st2 == 1 ? k_lds1 : k_lds2), st2 == 0 ? v_lds0 : (st2 == 1 ? v_lds1 : v_lds2));
+      // a wavefront whose 32 query rows all lie before this kv block has nothing to add (causal)
+      if (!CAUSAL || j * kKvBlock <= q_wave0 + kQWave - 1)
+        compute_tile(j, st == 0 ? k_lds0 : (st == 1 ? k_lds1 : k_lds2), st == 0 ? v_lds0 : (st == 1 ? v_lds1 : v_lds2),
+                     std::true_type());
+      stage_sync(j + 2 < n_tiles);
+    }
+  } else {
+    // Two stages: the copy of block j+1 is issued at the start of the step for block j and must have landed at its end.
+    issue_tile(0, k_lds0, v_lds0);
+    stage_sync(false);
+    if (n_tiles > 1) issue_tile(1, k_lds1, v_lds1);
+    compute_tile(0, k_lds0, v_lds0, std::true_type());
+    stage_sync(false);
+    int j = 1;
+    for (; j + 1 < n_plain && j + 2 < n_tiles; j += 2) {
+      issue_tile(j + 1, k_lds0, v_lds0);
+      compute_tile(j, k_lds1, v_lds1, std::false_type());
+      stage_sync(false);
+      issue_tile(j + 2, k_lds1, v_lds1);
+      compute_tile(j + 1, k_lds0, v_lds0, std::false_type());
+      stage_sync(false);
+    }
+    for (; j < n_tiles; ++j) {
+      const bool odd = j & 1;
+      if (j + 1 < n_tiles) issue_tile(j + 1, odd ? k_lds0 : k_lds1, odd ? v_lds0 : v_lds1);
+      if (!CAUSAL || j * kKvBlock <= q_wave0 + kQWave - 1)
+        compute_tile(j, odd ? k_lds1 : k_lds0, odd ? v_lds1 : v_lds0, std::true_type());
+      stage_sync(false);
+    }
   }
 
   // ---- epilogue: O / l, convert, store (reference csrc/flash_attention.cu:542-582) ----
@@ -498,7 +563,7 @@ extern "C" int fa8_fwd_validate(const Fa8FwdParams* p) {
   if (p->in_dtype != FA8_DTYPE_E4M3 && p->in_dtype != FA8_DTYPE_E5M2) return FA8_ERR_DTYPE;
   if (p->out_dtype != FA8_OUT_FP16 && p->out_dtype != FA8_OUT_E4M3) return FA8_ERR_DTYPE;
   if (p->v_layout != FA8_V_ROWS && p->v_layout != FA8_V_TRANSPOSED) return FA8_ERR_DTYPE;
-  if (p->head_dim != 64 && p->head_dim != 128) return FA8_ERR_HEAD_DIM;
+  if (p->head_dim % 32 != 0 || p->head_dim > 256) return FA8_ERR_HEAD_DIM;
   if (!(p->softmax_scale == p->softmax_scale) || std::isinf(p->softmax_scale)) return FA8_ERR_SCALE;
   const long long d = p->head_dim;
   const long long v_rows = p->v_layout == FA8_V_ROWS ? p->seqlen_k : d;
@@ -545,9 +610,20 @@ extern "C" int fa8_fwd(const Fa8FwdParams* p, void* hip_stream) {
   a.v_bs = p->v_batch_stride; a.v_hs = p->v_head_stride; a.v_rs = p->v_row_stride;
   a.o_bs = p->o_batch_stride; a.o_hs = p->o_head_stride; a.o_rs = p->o_row_stride;
   hipStream_t stream = (hipStream_t)hip_stream;
-  if (p->head_dim == 128)
-    return p->is_causal ? launch_types<128, true>(p, a, stream) : launch_types<128, false>(p, a, stream);
-  return p->is_causal ? launch_types<64, true>(p, a, stream) : launch_types<64, false>(p, a, stream);
+  switch (p->head_dim) {
+#define FA8_HEAD_DIM_CASE(D_) \
+  case D_: return p->is_causal ? launch_types<D_, true>(p, a, stream) : launch_types<D_, false>(p, a, stream)
+    FA8_HEAD_DIM_CASE(32);  // the head-dim buckets of the reference (csrc/static_switch.h:50-77)
+    FA8_HEAD_DIM_CASE(64);
+    FA8_HEAD_DIM_CASE(96);
+    FA8_HEAD_DIM_CASE(128);
+    FA8_HEAD_DIM_CASE(160);
+    FA8_HEAD_DIM_CASE(192);
+    FA8_HEAD_DIM_CASE(224);
+    FA8_HEAD_DIM_CASE(256);
+#undef FA8_HEAD_DIM_CASE
+    default: return FA8_ERR_HEAD_DIM;
+  }
 }
 
 extern "C" int fa8_query(int what) {
@@ -566,7 +642,7 @@ extern "C" const char* fa8_error_string(int code) {
     case FA8_OK: return "ok";
     case FA8_ERR_NULL: return "a required pointer is NULL";
     case FA8_ERR_SHAPE: return "bad shape (a size < 1, too many workgroups, or causal with seqlen_q != seqlen_k)";
-    case FA8_ERR_HEAD_DIM: return "head_dim must be 64 or 128";
+    case FA8_ERR_HEAD_DIM: return "head_dim must be a multiple of 32, at most 256";
     case FA8_ERR_STRIDE: return "a stride is smaller than the extent it spans";
     case FA8_ERR_ALIGN: return "q/k/v rows must be 16-byte aligned and o rows 8-byte aligned";
     case FA8_ERR_DTYPE: return "unknown in_dtype / out_dtype / v_layout code";

@@ -37,7 +37,7 @@ extern "C" {
 #define FA8_OK 0
 #define FA8_ERR_NULL (-1)        /* a required pointer is NULL */
 #define FA8_ERR_SHAPE (-2)       /* a size is < 1, or causal with seqlen_q != seqlen_k */
-#define FA8_ERR_HEAD_DIM (-3)    /* head_dim is not one of the compiled buckets (64, 128) */
+#define FA8_ERR_HEAD_DIM (-3)    /* head_dim is not a multiple of 32 in 32..256 */
 #define FA8_ERR_STRIDE (-4)      /* a stride is smaller than the extent it must span, or rows overlap */
 #define FA8_ERR_ALIGN (-5)       /* a base pointer or stride breaks the 16-byte row alignment the kernels load with (FA8_V_TRANSPOSED: also seqlen_k % 16 != 0) */
 #define FA8_ERR_DTYPE (-6)       /* unknown in_dtype/out_dtype/v_layout code */

@@ -71,9 +71,12 @@ def test_validate_rejects_bad_arguments():
     assert validate(p) == -2
     p = fa.make_params(q, k, v, o, True, 0.125); p.seqlen_k = 32
     assert validate(p) == -2  # causal needs seqlen_q == seqlen_k
-    for d in (32, 96, 256):
+    for d in (16, 48, 80, 288, 512):
         q2, k2, v2, o2 = cpu_tensors(d=d)
         assert validate(fa.make_params(q2, k2, v2, o2, False, 0.125)) == -3
+    for d in (32, 64, 96, 128, 160, 192, 224, 256):  # the reference's head-dim buckets (static_switch.h:50-77)
+        q2, k2, v2, o2 = cpu_tensors(d=d)
+        assert validate(fa.make_params(q2, k2, v2, o2, False, 0.125)) == 0
     p = fa.make_params(q, k, v, o, False, 0.125); p.k_row_stride = 32
     assert validate(p) == -4
     p = fa.make_params(q, k, v, o, False, 0.125); p.k_row_stride = 72
@@ -95,7 +98,7 @@ def test_validate_rejects_bad_arguments():
 
 def test_fa8_fwd_rejects_before_any_gpu_work():
     # invalid arguments must come back as negative codes even on a machine without a GPU
-    q, k, v, o = cpu_tensors(d=96)
+    q, k, v, o = cpu_tensors(d=80)
     p = fa.make_params(q, k, v, o, False, 0.125)
     assert fa.lib().fa8_fwd(ctypes.byref(p), None) == -3
 

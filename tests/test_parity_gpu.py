@@ -95,7 +95,7 @@ def test_cfg1_causal_full():
     check(q, k, v, inputs.softmax_scale(cfg), True, label="cfg1-causal")
 
 
-@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("d", [32, 64, 96, 128, 160, 192, 224, 256])
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("n", [1, 17, 64, 100, 128, 129, 200, 1000])
 def test_small_shapes(n, causal, d):
