@@ -25,7 +25,9 @@ EXT_PATH = os.path.join(_PKG_DIR, _EXT_NAME + sysconfig.get_config_var("EXT_SUFF
 FA8_DTYPE_E4M3, FA8_DTYPE_E5M2 = 0, 1
 FA8_OUT_FP16, FA8_OUT_E4M3 = 0, 1
 FA8_V_ROWS, FA8_V_TRANSPOSED = 0, 1
-FA8_QUERY_VERSION, FA8_QUERY_KV_BLOCK, FA8_QUERY_Q_BLOCK, FA8_QUERY_KV_ASCENDING, FA8_QUERY_THREADS = range(5)
+FA8_CAUSAL_TOP_LEFT, FA8_CAUSAL_BOTTOM_RIGHT = 0, 1
+(FA8_QUERY_VERSION, FA8_QUERY_KV_BLOCK, FA8_QUERY_Q_BLOCK, FA8_QUERY_KV_ASCENDING, FA8_QUERY_THREADS,
+ FA8_QUERY_PARAMS_SIZE) = range(6)
 FA8_EXPORTS = ("fa8_fwd_validate", "fa8_fwd", "fa8_query", "fa8_error_string")
 
 
@@ -41,6 +43,8 @@ class Fa8FwdParams(ctypes.Structure):
         ("k_batch_stride", ctypes.c_int64), ("k_head_stride", ctypes.c_int64), ("k_row_stride", ctypes.c_int64),
         ("v_batch_stride", ctypes.c_int64), ("v_head_stride", ctypes.c_int64), ("v_row_stride", ctypes.c_int64),
         ("o_batch_stride", ctypes.c_int64), ("o_head_stride", ctypes.c_int64), ("o_row_stride", ctypes.c_int64),
+        ("lse", ctypes.c_void_p), ("lse_batch_stride", ctypes.c_int64), ("lse_head_stride", ctypes.c_int64),
+        ("heads_k", ctypes.c_int32), ("causal_align", ctypes.c_int32),
     ]
 
 
@@ -90,8 +94,9 @@ def load_extension():
     return mod
 
 
-def make_params(q, k, v, o, is_causal, softmax_scale, v_transposed=False):
-    """Fill Fa8FwdParams from torch tensors (any device: only shapes, strides and pointers are read)."""
+def make_params(q, k, v, o, is_causal, softmax_scale, v_transposed=False, lse=None, causal_bottom_right=False):
+    """Fill Fa8FwdParams from torch tensors (any device: only shapes, strides and pointers are read).
+    k and v may have fewer heads than q (grouped-query attention); lse, if given, is a float32 [B,H,Nq] output."""
     import torch
     in_codes = {torch.float8_e4m3fn: FA8_DTYPE_E4M3, torch.float8_e5m2: FA8_DTYPE_E5M2}
     out_codes = {torch.float16: FA8_OUT_FP16, torch.float8_e4m3fn: FA8_OUT_E4M3}
@@ -119,16 +124,26 @@ def make_params(q, k, v, o, is_causal, softmax_scale, v_transposed=False):
         setattr(p, name + "_batch_stride", t.stride(0))
         setattr(p, name + "_head_stride", t.stride(1))
         setattr(p, name + "_row_stride", t.stride(2))
+    p.heads_k = k.shape[1]
+    p.causal_align = FA8_CAUSAL_BOTTOM_RIGHT if causal_bottom_right else FA8_CAUSAL_TOP_LEFT
+    if lse is not None:
+        if lse.dtype != torch.float32 or lse.dim() != 3 or lse.stride(2) != 1:
+            raise RuntimeError("lse must be a float32 [batch, heads, seqlen_q] tensor with contiguous rows")
+        p.lse, p.lse_batch_stride, p.lse_head_stride = lse.data_ptr(), lse.stride(0), lse.stride(1)
     return p
 
 
-def flash_attention_v2_cutlass(q, k, v, is_causal, softmax_scale, *, v_transposed=False, out_dtype=None):
+def flash_attention_v2_cutlass(q, k, v, is_causal, softmax_scale, *, v_transposed=False, out_dtype=None, return_lse=False,
+                               causal_bottom_right=False):
     """The reference operator (reference csrc/flash_attention.cu:639-668) through the C ABI.
 
     q, k: fp8 [B,H,N,d] on the GPU; v: [B,H,N,d] (or [B,H,d,N] with v_transposed=True, as the reference
     requires of its caller, test.py:71).  Returns [O], O fp16 [B,H,N,d] (out_dtype=torch.float8_e4m3fn
     gives the reference's fp8 O).  Runs on torch's current stream without synchronising.  Raises
     RuntimeError on bad arguments, like the reference's TORCH_CHECKs (include/attention_api.cuh:12-18).
+    Beyond the reference: k/v may have fewer heads than q (grouped-query attention), return_lse=True returns
+    [O, lse] with lse the float32 [B,H,Nq] log-sum-exp of the scaled logits, causal_bottom_right=True aligns the
+    causal diagonal with the last key when seqlen_q != seqlen_k.
     """
     import torch
     for name, t in (("q", q), ("k", k), ("v", v)):
@@ -139,22 +154,25 @@ def flash_attention_v2_cutlass(q, k, v, is_causal, softmax_scale, *, v_transpose
         if t.dim() != 4:
             raise RuntimeError(f"{name} must be 4-dimensional [batch, heads, seqlen, head_dim], got {t.dim()} dims")
     B, H, Nq, D = q.shape
-    Nk = k.shape[2]
-    if tuple(k.shape) != (B, H, Nk, D):
-        raise RuntimeError(f"k must be [{B}, {H}, seqlen_k, {D}], got {tuple(k.shape)}")
-    want_v = (B, H, D, Nk) if v_transposed else (B, H, Nk, D)
+    Nk, Hk = k.shape[2], k.shape[1]
+    if k.shape[0] != B or k.shape[3] != D:
+        raise RuntimeError(f"k must be [{B}, heads_k, seqlen_k, {D}], got {tuple(k.shape)}")
+    if Hk < 1 or H % Hk != 0:
+        raise RuntimeError(f"the number of q heads ({H}) must be a multiple of the number of k/v heads ({Hk})")
+    want_v = (B, Hk, D, Nk) if v_transposed else (B, Hk, Nk, D)
     if tuple(v.shape) != want_v:
         raise RuntimeError(f"v must be {list(want_v)}, got {tuple(v.shape)}")
     if k.device != q.device or v.device != q.device:
         raise RuntimeError("q, k and v must be on the same device")
     o = torch.empty((B, H, Nq, D), dtype=out_dtype or torch.float16, device=q.device)
-    p = make_params(q, k, v, o, is_causal, softmax_scale, v_transposed)
+    lse = torch.empty((B, H, Nq), dtype=torch.float32, device=q.device) if return_lse else None
+    p = make_params(q, k, v, o, is_causal, softmax_scale, v_transposed, lse, causal_bottom_right)
     with torch.cuda.device(q.device):
         stream = torch.cuda.current_stream(q.device).cuda_stream
         rc = lib().fa8_fwd(ctypes.byref(p), ctypes.c_void_p(stream))
     if rc != 0:
         raise RuntimeError(f"flash_attention_v2_cutlass: {error_string(rc)} (code {rc})")
-    return [o]
+    return [o, lse] if return_lse else [o]
 
 
 # Make `from attention_cutlass_fp8 import flash_attention_v2_cutlass` work once this package is imported

@@ -10,6 +10,9 @@
 //   * O is fp16 by default; `out_dtype=torch.float8_e4m3fn` gives the reference's fp8 O (:656);
 //   * the kernel runs on torch's current stream and the call does not synchronise the device (:661-665);
 //   * bad arguments and HIP errors raise RuntimeError instead of printf + exit (include/attention_api.cuh:20-29).
+// Additions the reference declares but never implements (csrc/flash.h:36-45,56): k/v may have fewer heads than q
+// (grouped-query attention), `return_lse=True` appends the fp32 log-sum-exp [B,H,Nq] to the returned list, and
+// `causal_bottom_right=True` aligns the causal diagonal with the last key when seqlen_q != seqlen_k.
 #include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <torch/extension.h>
@@ -31,7 +34,8 @@ void check_input(const torch::Tensor& t, const char* name) {
 
 std::vector<torch::Tensor> flash_attention_v2_cutlass(torch::Tensor q, torch::Tensor k, torch::Tensor v, bool is_causal,
                                                       float softmax_scale, bool v_transposed,
-                                                      c10::optional<at::ScalarType> out_dtype) {
+                                                      c10::optional<at::ScalarType> out_dtype, bool return_lse,
+                                                      bool causal_bottom_right) {
   check_input(q, "q");
   check_input(k, "k");
   check_input(v, "v");
@@ -41,14 +45,14 @@ std::vector<torch::Tensor> flash_attention_v2_cutlass(torch::Tensor q, torch::Te
   TORCH_CHECK(k.scalar_type() == in_type && v.scalar_type() == in_type, "q, k and v must have the same dtype");
   TORCH_CHECK(k.device() == q.device() && v.device() == q.device(), "q, k and v must be on the same device");
   const int64_t B = q.size(0), H = q.size(1), Nq = q.size(2), D = q.size(3);
-  const int64_t Nk = k.size(2);
-  TORCH_CHECK(k.size(0) == B && k.size(1) == H && k.size(3) == D, "k must be [", B, ", ", H, ", seqlen_k, ", D, "], got ",
-              k.sizes());
+  const int64_t Nk = k.size(2), Hk = k.size(1);
+  TORCH_CHECK(k.size(0) == B && k.size(3) == D, "k must be [", B, ", heads_k, seqlen_k, ", D, "], got ", k.sizes());
+  TORCH_CHECK(Hk >= 1 && H % Hk == 0, "the number of q heads (", H, ") must be a multiple of the number of k/v heads (", Hk, ")");
   if (v_transposed) {
-    TORCH_CHECK(v.size(0) == B && v.size(1) == H && v.size(2) == D && v.size(3) == Nk, "v (transposed) must be [", B, ", ",
-                H, ", ", D, ", ", Nk, "], got ", v.sizes());
+    TORCH_CHECK(v.size(0) == B && v.size(1) == Hk && v.size(2) == D && v.size(3) == Nk, "v (transposed) must be [", B, ", ",
+                Hk, ", ", D, ", ", Nk, "], got ", v.sizes());
   } else {
-    TORCH_CHECK(v.size(0) == B && v.size(1) == H && v.size(2) == Nk && v.size(3) == D, "v must be [", B, ", ", H, ", ", Nk,
+    TORCH_CHECK(v.size(0) == B && v.size(1) == Hk && v.size(2) == Nk && v.size(3) == D, "v must be [", B, ", ", Hk, ", ", Nk,
                 ", ", D, "], got ", v.sizes());
   }
   TORCH_CHECK(B >= 1 && H >= 1 && Nq >= 1 && Nk >= 1, "empty tensors are not supported");
@@ -57,8 +61,10 @@ std::vector<torch::Tensor> flash_attention_v2_cutlass(torch::Tensor q, torch::Te
   TORCH_CHECK(o_type == at::kHalf || o_type == at::kFloat8_e4m3fn, "out_dtype must be torch.float16 or torch.float8_e4m3fn");
 
   auto out = torch::empty({B, H, Nq, D}, q.options().dtype(o_type));
+  torch::Tensor lse;
+  if (return_lse) lse = torch::empty({B, H, Nq}, q.options().dtype(at::kFloat));
 
-  Fa8FwdParams p;
+  Fa8FwdParams p = {};
   p.q = q.data_ptr();
   p.k = k.data_ptr();
   p.v = v.data_ptr();
@@ -77,12 +83,20 @@ std::vector<torch::Tensor> flash_attention_v2_cutlass(torch::Tensor q, torch::Te
   p.k_batch_stride = k.stride(0); p.k_head_stride = k.stride(1); p.k_row_stride = k.stride(2);
   p.v_batch_stride = v.stride(0); p.v_head_stride = v.stride(1); p.v_row_stride = v.stride(2);
   p.o_batch_stride = out.stride(0); p.o_head_stride = out.stride(1); p.o_row_stride = out.stride(2);
+  p.heads_k = (int32_t)Hk;
+  p.causal_align = causal_bottom_right ? FA8_CAUSAL_BOTTOM_RIGHT : FA8_CAUSAL_TOP_LEFT;
+  if (return_lse) {
+    p.lse = lse.data_ptr();
+    p.lse_batch_stride = lse.stride(0);
+    p.lse_head_stride = lse.stride(1);
+  }
 
   // PyTorch-ROCm presents HIP devices under the "cuda" device type; these are its guard and stream for them.
   const c10::hip::HIPGuardMasqueradingAsCUDA device_guard(q.device());
   const hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(q.device().index()).stream();
   const int rc = fa8_fwd(&p, (void*)stream);
   TORCH_CHECK(rc == FA8_OK, "flash_attention_v2_cutlass: ", fa8_error_string(rc), " (code ", rc, ")");
+  if (return_lse) return {out, lse};
   return {out};
 }
 
@@ -91,6 +105,6 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("flash_attention_v2_cutlass", &flash_attention_v2_cutlass,
         "FP8 flash attention forward: fp8 q/k/v [B,H,N,d] -> [O] (fp16 by default)", py::arg("q"), py::arg("k"),
         py::arg("v"), py::arg("is_causal"), py::arg("softmax_scale"), py::kw_only(), py::arg("v_transposed") = false,
-        py::arg("out_dtype") = py::none());
+        py::arg("out_dtype") = py::none(), py::arg("return_lse") = false, py::arg("causal_bottom_right") = false);
   m.def("kv_block", []() { return fa8_query(FA8_QUERY_KV_BLOCK); }, "kv rows per online-softmax step of the kernel");
 }

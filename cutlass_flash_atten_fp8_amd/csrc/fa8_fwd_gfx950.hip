@@ -48,19 +48,23 @@ constexpr int kQBlock = 128;   // query rows per workgroup
 constexpr int kQWave = 32;     // query rows per wavefront
 constexpr int kKvBlock = 64;   // kv rows per online-softmax step
 constexpr int kThreads = 256;  // 4 wavefronts
-constexpr int kVersion = 1;
+constexpr int kVersion = 2;
 
 struct KernelArgs {
   const uint8_t* q;
   const uint8_t* k;
   const uint8_t* v;
   void* o;
+  float* lse;  // optional
   int heads, seqlen_q, seqlen_k, n_qblocks, bh_total;
+  int kv_group;      // q heads per k/v head
+  int causal_shift;  // key j is visible to query i when j <= i + causal_shift
   float scale_log2;  // softmax_scale * log2(e)
   long long q_bs, q_hs, q_rs;
   long long k_bs, k_hs, k_rs;
   long long v_bs, v_hs, v_rs;
   long long o_bs, o_hs, o_rs;
+  long long lse_bs, lse_hs;
 };
 
 // LDS row r (0..63) of a K tile holds kv row kv_of_lds_row(r) of the block.  With this order the 16
@@ -163,7 +167,9 @@ __device__ __forceinline__ void decode_block(const KernelArgs& a, int id, int& b
   int qi;
   if ((a.bh_total & 7) == 0) {
     const int xcd = id & 7, s = id >> 3;
-    bh = (s / a.n_qblocks) * 8 + xcd;
+    // grouped-query attention: an XCD takes a contiguous range of q heads, so the heads that share a k/v head follow
+    // each other on one XCD
+    bh = a.kv_group > 1 ? xcd * (a.bh_total >> 3) + s / a.n_qblocks : (s / a.n_qblocks) * 8 + xcd;
     qi = s % a.n_qblocks;
   } else {
     bh = id / a.n_qblocks;
@@ -209,8 +215,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
   const int q_wave0 = q0 + wave * kQWave;
   const int q_row = q_wave0 + qn;  // this lane's query row
   const uint8_t* qp = a.q + b * a.q_bs + hd * a.q_hs;
-  const uint8_t* kp = a.k + b * a.k_bs + hd * a.k_hs;
-  const uint8_t* vp = a.v + b * a.v_bs + hd * a.v_hs;
+  const int hd_kv = a.kv_group == 1 ? hd : hd / a.kv_group;  // grouped-query attention: several q heads per k/v head
+  const uint8_t* kp = a.k + b * a.k_bs + hd_kv * a.k_hs;
+  const uint8_t* vp = a.v + b * a.v_bs + hd_kv * a.v_hs;
   const float c = a.scale_log2;
 
   // ---- Q fragment (B operand of S^T = K Q^T): row q_row, bytes [64ks + 32h, +32) ----
@@ -310,11 +317,15 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
   constexpr int kVtTileStride = 32 * 64;  // LDS bytes between 32-row groups of the [d][64] tile
   constexpr int kTrStride = 8 * DP;  // LDS bytes between successive groups of 8 kv rows
 
-  const int n_tiles = CAUSAL ? (min(a.seqlen_k, q0 + kQBlock) + kKvBlock - 1) / kKvBlock
+  // Causal: key j is visible to query i when j <= i + shift (shift 0: the reference's rule, csrc/flash_attention.cu:62-64;
+  // shift = Nk - Nq aligns the diagonal with the bottom right corner).  At least block 0 is always walked (fully
+  // masked if need be), so a query that sees no key ends with l = 0 and an all-zero output row.
+  const int shift = CAUSAL ? a.causal_shift : 0;
+  const int n_tiles = CAUSAL ? max(1, (min(a.seqlen_k, q0 + kQBlock + shift) + kKvBlock - 1) / kKvBlock)
                              : (a.seqlen_k + kKvBlock - 1) / kKvBlock;
-  // Leading blocks that need no mask for any row of the workgroup: they end at or before the first query row
-  // (causal) and inside the kv range.  They are processed in pairs by the mask-free copy of the loop body.
-  const int n_plain = (CAUSAL ? min(q0, a.seqlen_k) : a.seqlen_k) / kKvBlock;
+  // Leading blocks that need no mask for any row of the workgroup: they end at or before the first query row's
+  // last visible key (causal) and inside the kv range.  They are processed by the mask-free copy of the loop body.
+  const int n_plain = (CAUSAL ? max(0, min(q0 + shift, a.seqlen_k)) : a.seqlen_k) / kKvBlock;
 
   v16f o_acc[kMTiles];
 #pragma unroll
@@ -344,7 +355,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
       }
     }
     // ---- causal / tail mask: register i of sub-tile t is kv row kv0 + 32h + 16t + i ----
-    const int kv_limit = CAUSAL ? min(q_row, kv_last) : kv_last;  // last kv this query attends to
+    const int kv_limit = CAUSAL ? min(q_row + shift, kv_last) : kv_last;  // last kv this query attends to
     if constexpr (kMasked) {
 #pragma unroll
       for (int t = 0; t < 2; ++t)
@@ -465,7 +476,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
       if (j + 2 < n_tiles)
         issue_tile(j + 2, st2 == 0 ? k_lds0 : (st2 == 1 ? k_lds1 : k_lds2), st2 == 0 ? v_lds0 : (st2 == 1 ? v_lds1 : v_lds2));
       // a wavefront whose 32 query rows all lie before this kv block has nothing to add (causal)
-      if (!CAUSAL || j * kKvBlock <= q_wave0 + kQWave - 1)
+      if (!CAUSAL || j * kKvBlock <= q_wave0 + kQWave - 1 + shift)
         compute_tile(j, st == 0 ? k_lds0 : (st == 1 ? k_lds1 : k_lds2), st == 0 ? v_lds0 : (st == 1 ? v_lds1 : v_lds2),
                      std::true_type());
       stage_sync(j + 2 < n_tiles);
@@ -489,7 +500,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
     for (; j < n_tiles; ++j) {
       const bool odd = j & 1;
       if (j + 1 < n_tiles) issue_tile(j + 1, odd ? k_lds0 : k_lds1, odd ? v_lds0 : v_lds1);
-      if (!CAUSAL || j * kKvBlock <= q_wave0 + kQWave - 1)
+      if (!CAUSAL || j * kKvBlock <= q_wave0 + kQWave - 1 + shift)
         compute_tile(j, odd ? k_lds1 : k_lds0, odd ? v_lds1 : v_lds0, std::true_type());
       stage_sync(false);
     }
@@ -498,6 +509,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
   // ---- epilogue: O / l, convert, store (reference csrc/flash_attention.cu:542-582) ----
   const float l_tot = lane32_sum(l_run);
   const float inv = (l_tot == 0.f || l_tot != l_tot) ? 1.f : 1.f / l_tot;
+  // log-sum-exp of the scaled logits of the row (natural log), -inf for a row that saw no key; the reference reserves
+  // the output but never writes it (csrc/flash.h:56, csrc/flash_attention.cu:658-659)
+  if (a.lse != nullptr && h == 0 && q_row < a.seqlen_q) {
+    const float lse = l_tot > 0.f ? (m_run * c + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f : (l_tot == 0.f ? -INFINITY : l_tot);
+    a.lse[b * a.lse_bs + hd * a.lse_hs + q_row] = lse;
+  }
   if (q_row < a.seqlen_q) {
     // register i = 4a2 + b2 of tile mt is head-dim column 32mt + 8a2 + 4h + b2
     if constexpr (OUT == FA8_OUT_FP16) {
@@ -558,7 +575,8 @@ extern "C" int fa8_fwd_validate(const Fa8FwdParams* p) {
   if (p == nullptr || p->q == nullptr || p->k == nullptr || p->v == nullptr || p->o == nullptr) return FA8_ERR_NULL;
   if (p->batch < 1 || p->heads < 1 || p->seqlen_q < 1 || p->seqlen_k < 1 || p->head_dim < 1) return FA8_ERR_SHAPE;
   if (p->is_causal != 0 && p->is_causal != 1) return FA8_ERR_SHAPE;
-  if (p->is_causal && p->seqlen_q != p->seqlen_k) return FA8_ERR_SHAPE;
+  if (p->heads_k < 0 || (p->heads_k > 0 && p->heads % p->heads_k != 0)) return FA8_ERR_SHAPE;
+  if (p->causal_align != FA8_CAUSAL_TOP_LEFT && p->causal_align != FA8_CAUSAL_BOTTOM_RIGHT) return FA8_ERR_DTYPE;
   if ((long long)p->batch * p->heads > 0x7fffffffLL / ((p->seqlen_q + kQBlock - 1) / kQBlock)) return FA8_ERR_SHAPE;
   if (p->in_dtype != FA8_DTYPE_E4M3 && p->in_dtype != FA8_DTYPE_E5M2) return FA8_ERR_DTYPE;
   if (p->out_dtype != FA8_OUT_FP16 && p->out_dtype != FA8_OUT_E4M3) return FA8_ERR_DTYPE;
@@ -583,6 +601,10 @@ extern "C" int fa8_fwd_validate(const Fa8FwdParams* p) {
   for (long long s : o_strides)
     if ((s * o_elem) % 8 != 0) return FA8_ERR_ALIGN;
   if ((uintptr_t)p->o % 8 != 0) return FA8_ERR_ALIGN;
+  if (p->lse != nullptr) {
+    if (!span_ok(p->lse_head_stride, p->seqlen_q) || !span_ok(p->lse_batch_stride, 1)) return FA8_ERR_STRIDE;
+    if ((uintptr_t)p->lse % 4 != 0) return FA8_ERR_ALIGN;
+  }
   // the kernels address k and v of one head with 32-bit byte offsets
   if ((long long)p->seqlen_k * p->k_row_stride > 0x7fffffffLL || v_rows * p->v_row_stride > 0x7fffffffLL) return FA8_ERR_SHAPE;
   // transposed v is read in 16-byte chunks along kv
@@ -599,6 +621,10 @@ extern "C" int fa8_fwd(const Fa8FwdParams* p, void* hip_stream) {
   a.k = (const uint8_t*)p->k;
   a.v = (const uint8_t*)p->v;
   a.o = p->o;
+  a.lse = (float*)p->lse;
+  a.lse_bs = p->lse_batch_stride; a.lse_hs = p->lse_head_stride;
+  a.kv_group = p->heads_k > 0 ? p->heads / p->heads_k : 1;
+  a.causal_shift = p->causal_align == FA8_CAUSAL_BOTTOM_RIGHT ? p->seqlen_k - p->seqlen_q : 0;
   a.heads = p->heads;
   a.seqlen_q = p->seqlen_q;
   a.seqlen_k = p->seqlen_k;
@@ -633,6 +659,7 @@ extern "C" int fa8_query(int what) {
     case FA8_QUERY_Q_BLOCK: return kQBlock;
     case FA8_QUERY_KV_ASCENDING: return 1;
     case FA8_QUERY_THREADS: return kThreads;
+    case FA8_QUERY_PARAMS_SIZE: return (int)sizeof(Fa8FwdParams);
     default: return -1;
   }
 }
@@ -641,11 +668,11 @@ extern "C" const char* fa8_error_string(int code) {
   switch (code) {
     case FA8_OK: return "ok";
     case FA8_ERR_NULL: return "a required pointer is NULL";
-    case FA8_ERR_SHAPE: return "bad shape (a size < 1, too many workgroups, or causal with seqlen_q != seqlen_k)";
+    case FA8_ERR_SHAPE: return "bad shape (a size < 1, too many workgroups, or heads not a multiple of heads_k)";
     case FA8_ERR_HEAD_DIM: return "head_dim must be a multiple of 32, at most 256";
     case FA8_ERR_STRIDE: return "a stride is smaller than the extent it spans";
     case FA8_ERR_ALIGN: return "q/k/v rows must be 16-byte aligned and o rows 8-byte aligned";
-    case FA8_ERR_DTYPE: return "unknown in_dtype / out_dtype / v_layout code";
+    case FA8_ERR_DTYPE: return "unknown in_dtype / out_dtype / v_layout / causal_align code";
     case FA8_ERR_UNSUPPORTED: return "this build has no kernel for the requested combination";
     case FA8_ERR_SCALE: return "softmax_scale must be finite";
     default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown fa8 error code";

@@ -33,14 +33,18 @@ extern "C" {
 #define FA8_V_ROWS 0       /* v is [B,H,Nk,d]: same as k */
 #define FA8_V_TRANSPOSED 1 /* v is [B,H,d,Nk]: what the reference requires of its caller (test.py:71) */
 
+/* which keys a query sees when is_causal (matters only when seqlen_q != seqlen_k) */
+#define FA8_CAUSAL_TOP_LEFT 0     /* key j <= query i: the reference's rule (csrc/flash_attention.cu:62-64, loop bound :458) */
+#define FA8_CAUSAL_BOTTOM_RIGHT 1 /* key j <= i + seqlen_k - seqlen_q: the last query sees every key (decode, chunked prefill) */
+
 /* error codes (all negative) */
 #define FA8_OK 0
 #define FA8_ERR_NULL (-1)        /* a required pointer is NULL */
-#define FA8_ERR_SHAPE (-2)       /* a size is < 1, or causal with seqlen_q != seqlen_k */
+#define FA8_ERR_SHAPE (-2)       /* a size is < 1, the grid would overflow, or heads is not a multiple of heads_k */
 #define FA8_ERR_HEAD_DIM (-3)    /* head_dim is not a multiple of 32 in 32..256 */
 #define FA8_ERR_STRIDE (-4)      /* a stride is smaller than the extent it must span, or rows overlap */
 #define FA8_ERR_ALIGN (-5)       /* a base pointer or stride breaks the 16-byte row alignment the kernels load with (FA8_V_TRANSPOSED: also seqlen_k % 16 != 0) */
-#define FA8_ERR_DTYPE (-6)       /* unknown in_dtype/out_dtype/v_layout code */
+#define FA8_ERR_DTYPE (-6)       /* unknown in_dtype/out_dtype/v_layout/causal_align code */
 #define FA8_ERR_UNSUPPORTED (-7) /* a valid combination that this build has no kernel for */
 #define FA8_ERR_SCALE (-8)       /* softmax_scale is NaN or infinite */
 
@@ -53,15 +57,15 @@ extern "C" {
  */
 typedef struct Fa8FwdParams {
   const void* q; /* [B,H,Nq,d] fp8 */
-  const void* k; /* [B,H,Nk,d] fp8 */
-  const void* v; /* [B,H,Nk,d] fp8 (FA8_V_ROWS) or [B,H,d,Nk] (FA8_V_TRANSPOSED) */
+  const void* k; /* [B,Hk,Nk,d] fp8; Hk = heads_k (or heads) */
+  const void* v; /* [B,Hk,Nk,d] fp8 (FA8_V_ROWS) or [B,Hk,d,Nk] (FA8_V_TRANSPOSED) */
   void* o;       /* [B,H,Nq,d] fp16 or e4m3 */
   int32_t batch;
   int32_t heads;
   int32_t seqlen_q;
   int32_t seqlen_k;
   int32_t head_dim;
-  int32_t is_causal; /* 0/1; causal needs seqlen_q == seqlen_k (as csrc/flash_attention.cu:458 assumes) */
+  int32_t is_causal; /* 0/1 */
   int32_t in_dtype;  /* FA8_DTYPE_* */
   int32_t out_dtype; /* FA8_OUT_* */
   int32_t v_layout;  /* FA8_V_* */
@@ -70,6 +74,18 @@ typedef struct Fa8FwdParams {
   int64_t k_batch_stride, k_head_stride, k_row_stride;
   int64_t v_batch_stride, v_head_stride, v_row_stride; /* row = kv row (FA8_V_ROWS) or d row (FA8_V_TRANSPOSED) */
   int64_t o_batch_stride, o_head_stride, o_row_stride;
+  /* ---- library version 2 (fa8_query(FA8_QUERY_VERSION) >= 2); all-zero = the behaviour of version 1 ---- */
+  /* Optional output (NULL: not wanted): lse[b,h,i] = log(sum_j exp(softmax_scale * S[i,j])) over the keys query i sees,
+   * fp32 [B,H,Nq], rows contiguous; -inf for a query that sees no key.  It is what merges partial results of a kv-split
+   * (context-parallel) run.  The reference reserves softmax_lse_ptr but always passes nullptr
+   * (csrc/flash.h:56, csrc/flash_attention.cu:658-659). */
+  void* lse;
+  int64_t lse_batch_stride, lse_head_stride;
+  /* Grouped-query / multi-query attention: number of k/v heads; 0 (or == heads) = one per q head.  heads must be a
+   * multiple; q head h reads k/v head h / (heads / heads_k).  (Reference fields k_head, h_h_k_ratio, csrc/flash.h:36-45:
+   * declared, never used by its kernel.) */
+  int32_t heads_k;
+  int32_t causal_align; /* FA8_CAUSAL_* */
 } Fa8FwdParams;
 
 /*
@@ -93,6 +109,7 @@ int fa8_fwd(const Fa8FwdParams* p, void* hip_stream);
 #define FA8_QUERY_Q_BLOCK 2       /* q rows per workgroup */
 #define FA8_QUERY_KV_ASCENDING 3  /* 1: kv blocks are visited in ascending order (as the reference loop :468) */
 #define FA8_QUERY_THREADS 4       /* threads per workgroup */
+#define FA8_QUERY_PARAMS_SIZE 5   /* sizeof(Fa8FwdParams) of the library: a caller built against another layout can tell */
 int fa8_query(int what);
 
 /* Static, human-readable text for a return code of this library (never NULL). */

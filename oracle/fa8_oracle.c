@@ -24,7 +24,10 @@
  *     codes, cross-checked against torch's CPU cast;
  *   - fa8o_fwd_rows: an independent numpy restatement, closed-form known answers (dominant logit, equal
  *     keys, scale = 0, causal row 0, constant V), brute-force fp64 triple loops on tiny inputs, and
- *     equality with fp64 softmax attention when P quantisation is switched off.
+ *     equality with fp64 softmax attention when P quantisation is switched off;
+ *   - the extensions beyond the reference's kernel (heads_k, causal_shift, lse; tests/test_oracle_extensions.py):
+ *     grouped-query attention equals multi-head attention on repeated k/v heads, the log-sum-exp equals a direct
+ *     fp64 logsumexp of the scaled logits, a shifted causal mask equals a brute-force boolean mask.
  * Not pinned (hardware details no CPU reproduces, both far below the tolerance): the accumulation order
  * inside the sm_89 tensor core and the ulp behaviour of __expf under --use_fast_math.
  */
@@ -162,7 +165,25 @@ typedef struct Fa8OracleArgs {
   /* Optional rounding-flip allowance, see oracle_row.  flip_allow is float [B,H,n_rows] or NULL. */
   float* flip_allow;
   float logit_rel_err; /* bound on |S_device - S_exact| / sum_k |q_k k_k| of the matrix core being checked */
+  /* Extensions the reference declares but does not implement (csrc/flash.h:36-45,56). */
+  int32_t heads_k;      /* k/v heads (0 = heads); q head h uses k/v head h / (heads / heads_k) */
+  int32_t causal_shift; /* causal: column j is visible to row i when j <= i + causal_shift (reference: 0, :62-64) */
+  float* lse;           /* optional float [B,H,n_rows]: scale*m + log(l) of the row, -inf when the row sees no column */
 } Fa8OracleArgs;
+
+/* number of leading columns row i sees */
+static int visible_columns(const Fa8OracleArgs* a, int i) {
+  if (!a->is_causal) return a->seqlen_k;
+  const long long e = (long long)i + 1 + a->causal_shift;
+  return e < 0 ? 0 : (e < a->seqlen_k ? (int)e : a->seqlen_k);
+}
+
+/* index of the (batch, k/v head) pair that (batch, q head) pair bh reads */
+static int kv_head_of(const Fa8OracleArgs* a, int bh) {
+  const int hk = a->heads_k > 0 ? a->heads_k : a->heads;
+  const int b = bh / a->heads, h = bh % a->heads;
+  return b * hk + h / (a->heads / hk);
+}
 
 /* 256-entry decode tables filled from the closed forms above (idempotent, so concurrent first calls are harmless). */
 static float g_lut[2][256];
@@ -209,7 +230,7 @@ static float tie_distance(float p, int mbits, int emin, float* quantum) {
 
 /* One query row.  kf/vf are the dequantised K [Nk,d] and V [Nk,d] of this head; p is scratch [kv_block]. */
 static void oracle_row(const Fa8OracleArgs* a, const float* qrow, const float* kf, const float* vf, int i, float* p,
-                       float* acc /* [d] */, float* flip_allow) {
+                       float* acc /* [d] */, float* flip_allow, float* lse) {
   /* flip_allow (optional): P is rounded to 3 (e4m3) or 2 (e5m2) mantissa bits, so a device whose logits differ
    * from the exact ones by a few 1e-5 of sum|q_k k_k| (matrix cores do not accumulate in IEEE fp32) can round a
    * P that lies next to a rounding boundary the other way: a legitimate one-quantum difference that changes
@@ -224,7 +245,7 @@ static void oracle_row(const Fa8OracleArgs* a, const float* qrow, const float* k
   for (int x = 0; x < d; ++x) acc[x] = 0.0f;
   /* Reference loop bound (:458): every block that starts before the end of the row's q block.  Blocks that
    * start after column i are fully masked for this row (m, l and O unchanged), so the loop may stop at j0 <= i. */
-  const int j_end = a->is_causal ? (i + 1 < nk ? i + 1 : nk) : nk; /* columns [0, j_end) are visible */
+  const int j_end = visible_columns(a, i); /* columns [0, j_end) are visible */
   for (int j0 = 0; j0 < j_end; j0 += bc) {
     const int jn = j0 + bc < nk ? j0 + bc : nk; /* the block covers columns [j0, jn) */
     float bmax = -INFINITY;
@@ -274,13 +295,14 @@ static void oracle_row(const Fa8OracleArgs* a, const float* qrow, const float* k
   const float inv = (l == 0.0f || l != l) ? 1.0f : 1.0f / l; /* :545-553 */
   for (int x = 0; x < d; ++x) acc[x] *= inv;
   if (flip_allow) *flip_allow = allow * inv;
+  if (lse) *lse = l > 0.0f ? (float)((double)m * (double)scale + log((double)l)) : (l == 0.0f ? -INFINITY : l);
 }
 
 static void dequant_head(const Fa8OracleArgs* a, int bh, float* kf, float* vf) {
   const int nk = a->seqlen_k, d = a->head_dim;
   const float* lut = g_lut[a->in_dtype == FA8O_E5M2 ? FA8O_E5M2 : FA8O_E4M3];
-  const uint8_t* kq = a->k + (size_t)bh * nk * d;
-  const uint8_t* vq = a->v + (size_t)bh * nk * d;
+  const uint8_t* kq = a->k + (size_t)kv_head_of(a, bh) * nk * d;
+  const uint8_t* vq = a->v + (size_t)kv_head_of(a, bh) * nk * d;
   if (kf)
     for (size_t t = 0; t < (size_t)nk * d; ++t) kf[t] = lut[kq[t]];
   for (int j = 0; j < nk; ++j)
@@ -295,6 +317,7 @@ static void dequant_head(const Fa8OracleArgs* a, int bh, float* kf, float* vf) {
 int fa8o_fwd_rows(const Fa8OracleArgs* a, const int32_t* rows, int32_t n_rows) {
   const int B = a->batch, H = a->heads, nq = a->seqlen_q, nk = a->seqlen_k, d = a->head_dim;
   if (B < 1 || H < 1 || nq < 1 || nk < 1 || d < 1 || a->kv_block < 1) return -1;
+  if (a->heads_k < 0 || (a->heads_k > 0 && H % a->heads_k != 0)) return -1;
   const int nr = rows ? n_rows : nq;
   if (nr < 1) return -1;
   if (rows)
@@ -329,7 +352,8 @@ int fa8o_fwd_rows(const Fa8OracleArgs* a, const int32_t* rows, int32_t n_rows) {
         const int i = rows ? rows[r] : r;
         const uint8_t* qq = a->q + ((size_t)bh * nq + i) * d;
         for (int x = 0; x < d; ++x) qrow[x] = lut[qq[x]];
-        oracle_row(a, qrow, kf, vf, i, p, acc, a->flip_allow ? a->flip_allow + (size_t)bh * nr + r : NULL);
+        oracle_row(a, qrow, kf, vf, i, p, acc, a->flip_allow ? a->flip_allow + (size_t)bh * nr + r : NULL,
+                   a->lse ? a->lse + (size_t)bh * nr + r : NULL);
         const size_t o0 = ((size_t)bh * nr + r) * d;
         if (a->out_dtype == FA8O_OUT_FP16) {
           uint16_t* o = (uint16_t*)a->o;
@@ -353,6 +377,7 @@ int fa8o_fwd_rows(const Fa8OracleArgs* a, const int32_t* rows, int32_t n_rows) {
 int fa8o_attention_f64(const Fa8OracleArgs* a, const int32_t* rows, int32_t n_rows, double* o) {
   const int B = a->batch, H = a->heads, nq = a->seqlen_q, nk = a->seqlen_k, d = a->head_dim;
   if (B < 1 || H < 1 || nq < 1 || nk < 1 || d < 1) return -1;
+  if (a->heads_k < 0 || (a->heads_k > 0 && H % a->heads_k != 0)) return -1;
   const int nr = rows ? n_rows : nq;
   if (nr < 1) return -1;
   if (rows)
@@ -383,7 +408,7 @@ int fa8o_attention_f64(const Fa8OracleArgs* a, const int32_t* rows, int32_t n_ro
         if (failed) continue;
         const int i = rows ? rows[r] : r;
         const uint8_t* qq = a->q + ((size_t)bh * nq + i) * d;
-        const int j_end = a->is_causal ? (i + 1 < nk ? i + 1 : nk) : nk;
+        const int j_end = visible_columns(a, i);
         double mx = -INFINITY;
         for (int j = 0; j < j_end; ++j) {
           double acc = 0.0;
@@ -398,7 +423,7 @@ int fa8o_attention_f64(const Fa8OracleArgs* a, const int32_t* rows, int32_t n_ro
         }
         double* orow = o + ((size_t)bh * nr + r) * d;
         for (int x = 0; x < d; ++x) orow[x] = 0.0;
-        for (int j = 0; j < j_end; ++j) {
+        for (int j = 0; j < j_end; ++j) { /* a row that sees no column stays all zero */
           const double w = s[j] / den;
           for (int x = 0; x < d; ++x) orow[x] += w * (double)vf[(size_t)j * d + x];
         }

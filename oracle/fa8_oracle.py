@@ -25,6 +25,7 @@ class _Args(ctypes.Structure):
         ("kv_block", ctypes.c_int32), ("in_dtype", ctypes.c_int32), ("out_dtype", ctypes.c_int32),
         ("v_transposed", ctypes.c_int32), ("quantize_p", ctypes.c_int32), ("exp2_form", ctypes.c_int32),
         ("softmax_scale", ctypes.c_float), ("flip_allow", ctypes.c_void_p), ("logit_rel_err", ctypes.c_float),
+        ("heads_k", ctypes.c_int32), ("causal_shift", ctypes.c_int32), ("lse", ctypes.c_void_p),
     ]
 
 
@@ -71,14 +72,15 @@ def _prep(q, k, v, v_transposed):
     v = np.ascontiguousarray(v, dtype=np.uint8)
     assert q.ndim == 4 and k.ndim == 4 and v.ndim == 4
     B, H, nq, d = q.shape
-    nk = k.shape[2]
-    assert k.shape == (B, H, nk, d)
-    assert v.shape == ((B, H, d, nk) if v_transposed else (B, H, nk, d))
-    return q, k, v, B, H, nq, nk, d
+    nk, hk = k.shape[2], k.shape[1]
+    assert k.shape == (B, hk, nk, d) and H % hk == 0
+    assert v.shape == ((B, hk, d, nk) if v_transposed else (B, hk, nk, d))
+    return q, k, v, B, H, nq, nk, d, hk
 
 
 def forward(q, k, v, scale, causal=False, kv_block=64, rows=None, in_dtype=E4M3, out_dtype=OUT_FP16,
-            v_transposed=False, quantize_p=True, exp2_form=False, logit_rel_err=None):
+            v_transposed=False, quantize_p=True, exp2_form=False, logit_rel_err=None, causal_bottom_right=False,
+            return_lse=False):
     """The reference pipeline on uint8 views of fp8 q/k/v [B,H,N,d].
 
     Returns [B,H,n_rows,d] as float16 (OUT_FP16), uint8 e4m3 codes (OUT_E4M3) or float32 (OUT_F32).
@@ -86,32 +88,39 @@ def forward(q, k, v, scale, causal=False, kv_block=64, rows=None, in_dtype=E4M3,
     logit_rel_err: when given, also returns flip_allow float32 [B,H,n_rows]: how much O[row,:] may legitimately
     move because some P sits within reach of an fp8 rounding boundary for a device whose logits are accurate
     to logit_rel_err * sum_k|q_k k_k| (see oracle_row in fa8_oracle.c).
+    k and v may have fewer heads than q (grouped-query attention).  causal_bottom_right: column j is visible to row i
+    when j <= i + Nk - Nq instead of j <= i.  return_lse: also return float32 [B,H,n_rows], scale*rowmax + log(rowsum).
+    The result is res, or (res, allow), (res, lse), (res, allow, lse) in that order.
     """
-    q, k, v, B, H, nq, nk, d = _prep(q, k, v, v_transposed)
+    q, k, v, B, H, nq, nk, d, hk = _prep(q, k, v, v_transposed)
     rows_arr = None if rows is None else np.ascontiguousarray(rows, dtype=np.int32)
     nr = nq if rows_arr is None else int(rows_arr.shape[0])
     np_dtype = {OUT_FP16: np.uint16, OUT_E4M3: np.uint8, OUT_F32: np.float32}[out_dtype]
     o = np.zeros((B, H, nr, d), dtype=np_dtype)
     allow = None if logit_rel_err is None else np.zeros((B, H, nr), dtype=np.float32)
+    lse = np.zeros((B, H, nr), dtype=np.float32) if return_lse else None
     a = _Args(q.ctypes.data, k.ctypes.data, v.ctypes.data, o.ctypes.data, B, H, nq, nk, d, int(bool(causal)),
               int(kv_block), int(in_dtype), int(out_dtype), int(bool(v_transposed)), int(bool(quantize_p)),
               int(bool(exp2_form)), float(scale), None if allow is None else allow.ctypes.data,
-              0.0 if logit_rel_err is None else float(logit_rel_err))
+              0.0 if logit_rel_err is None else float(logit_rel_err), hk, nk - nq if causal_bottom_right else 0,
+              None if lse is None else lse.ctypes.data)
     rc = lib().fa8o_fwd_rows(ctypes.byref(a), None if rows_arr is None else rows_arr.ctypes.data, nr)
     if rc != 0:
         raise RuntimeError(f"fa8o_fwd_rows failed with {rc}")
     res = o.view(np.float16) if out_dtype == OUT_FP16 else o
-    return res if allow is None else (res, allow)
+    extra = tuple(x for x in (allow, lse) if x is not None)
+    return (res,) + extra if extra else res
 
 
-def attention_f64(q, k, v, scale, causal=False, rows=None, in_dtype=E4M3, v_transposed=False):
+def attention_f64(q, k, v, scale, causal=False, rows=None, in_dtype=E4M3, v_transposed=False, causal_bottom_right=False):
     """Exact fp64 softmax attention on the dequantised inputs; float64 [B,H,n_rows,d]."""
-    q, k, v, B, H, nq, nk, d = _prep(q, k, v, v_transposed)
+    q, k, v, B, H, nq, nk, d, hk = _prep(q, k, v, v_transposed)
     rows_arr = None if rows is None else np.ascontiguousarray(rows, dtype=np.int32)
     nr = nq if rows_arr is None else int(rows_arr.shape[0])
     o = np.zeros((B, H, nr, d), dtype=np.float64)
     a = _Args(q.ctypes.data, k.ctypes.data, v.ctypes.data, None, B, H, nq, nk, d, int(bool(causal)), 64,
-              int(in_dtype), OUT_F32, int(bool(v_transposed)), 0, 0, float(scale), None, 0.0)
+              int(in_dtype), OUT_F32, int(bool(v_transposed)), 0, 0, float(scale), None, 0.0, hk,
+              nk - nq if causal_bottom_right else 0, None)
     rc = lib().fa8o_attention_f64(ctypes.byref(a), None if rows_arr is None else rows_arr.ctypes.data, nr,
                                   o.ctypes.data)
     if rc != 0:

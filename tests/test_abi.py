@@ -36,6 +36,8 @@ def test_library_exports_every_declared_symbol():
 def test_query_values():
     assert fa.query(fa.FA8_QUERY_VERSION) >= 1
     assert fa.query(fa.FA8_QUERY_KV_BLOCK) in (64, 128)
+    assert fa.query(fa.FA8_QUERY_PARAMS_SIZE) == ctypes.sizeof(fa.Fa8FwdParams)  # the ctypes mirror has the C layout
+    assert fa.query(fa.FA8_QUERY_VERSION) >= 2
     assert fa.query(fa.FA8_QUERY_Q_BLOCK) % 32 == 0
     assert fa.query(fa.FA8_QUERY_KV_ASCENDING) == 1
     assert fa.query(fa.FA8_QUERY_THREADS) % 64 == 0
@@ -70,7 +72,25 @@ def test_validate_rejects_bad_arguments():
     p = fa.make_params(q, k, v, o, False, 0.125); p.seqlen_k = 0
     assert validate(p) == -2
     p = fa.make_params(q, k, v, o, True, 0.125); p.seqlen_k = 32
-    assert validate(p) == -2  # causal needs seqlen_q == seqlen_k
+    assert validate(p) == 0  # causal with seqlen_q != seqlen_k: top-left aligned by default
+    p.causal_align = fa.FA8_CAUSAL_BOTTOM_RIGHT
+    assert validate(p) == 0
+    p.causal_align = 2
+    assert validate(p) == -6
+    p = fa.make_params(q, k, v, o, False, 0.125); p.heads_k = 3  # 2 q heads
+    assert validate(p) == -2
+    p.heads_k = -1
+    assert validate(p) == -2
+    for hk in (0, 1, 2):
+        p.heads_k = hk
+        assert validate(p) == 0
+    lse = torch.zeros((1, 2, 64), dtype=torch.float32)
+    p = fa.make_params(q, k, v, o, False, 0.125, lse=lse)
+    assert validate(p) == 0
+    p.lse_head_stride = 63
+    assert validate(p) == -4
+    p = fa.make_params(q, k, v, o, False, 0.125, lse=lse); p.lse = p.lse + 2
+    assert validate(p) == -5
     for d in (16, 48, 80, 288, 512):
         q2, k2, v2, o2 = cpu_tensors(d=d)
         assert validate(fa.make_params(q2, k2, v2, o2, False, 0.125)) == -3

@@ -192,9 +192,9 @@ def test_error_paths_raise_and_launch_nothing():
         ext.flash_attention_v2_cutlass(q.half(), q.half(), q.half(), False, 0.1)
     with pytest.raises(RuntimeError, match="float8"):
         ext.flash_attention_v2_cutlass(*(t.view(torch.uint8).view(torch.float8_e4m3fnuz) for t in (q, q, q)), False, 0.1)
-    k_short = rand_fp8((1, 2, 64, 128), 32).to(DEV)
-    with pytest.raises(RuntimeError):  # causal needs seqlen_q == seqlen_k
-        ext.flash_attention_v2_cutlass(q, k_short, k_short, True, 0.1)
+    k3 = rand_fp8((1, 3, 128, 128), 32).to(DEV)
+    with pytest.raises(RuntimeError, match="multiple"):  # 2 q heads over 3 k/v heads
+        ext.flash_attention_v2_cutlass(q, k3, k3, True, 0.1)
     with pytest.raises(RuntimeError, match="finite"):
         ext.flash_attention_v2_cutlass(q, q, q, False, float("nan"))
     q100 = rand_fp8((1, 2, 100, 128), 33).to(DEV)
@@ -202,6 +202,7 @@ def test_error_paths_raise_and_launch_nothing():
         ext.flash_attention_v2_cutlass(q100, q100, q100.transpose(2, 3).contiguous(), False, 0.1, v_transposed=True)
     torch.cuda.synchronize()
     # seqlen_q != seqlen_k is fine without the causal mask
+    k_short = rand_fp8((1, 2, 64, 128), 34).to(DEV)
     o = ext.flash_attention_v2_cutlass(q, k_short, k_short, False, 0.1)[0]
     ref = fo.forward(u8(q), u8(k_short), u8(k_short), 0.1, exp2_form=True).astype(np.float32)
     assert np.abs(o.float().cpu().numpy() - ref).mean() <= 2e-3
