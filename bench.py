@@ -23,7 +23,8 @@ HBM_PEAK_GBPS = 8000.0
 
 # HBM bytes per launch of the headline workload read by rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), each scaled by
 # what the same counter reads for a plain copy kernel of known size; see profiles/.  None until measured.
-MEASURED_TRAFFIC_BYTES = {"cfg3": 168.0e6}  # profiles/fa8_fwd_kernel_d128_cfg3_headline.md, section 3
+MEASURED_TRAFFIC_BYTES = {"cfg3": 168.0e6,  # profiles/fa8_fwd_kernel_d128_cfg3_headline.md, section 3
+                          "cfg2": 21.2e6, "cfg4": 173.2e6, "cfg5": 103.1e6}  # profiles/fa8_fwd_kernel_cfg2_cfg4_cfg5.md
 
 
 # cutlass fp8 milliseconds published by the reference (benchmark.png, rows in the order of test.py:95-100; Ada sm_89,
