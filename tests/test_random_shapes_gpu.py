@@ -1,0 +1,63 @@
+"""GPU parity on a seeded random sweep over the whole argument space of the operator: head dim, k/v head count, both
+sequence lengths, causal mask and its alignment, v layout, input type, output type.  Gate as in the other parity tests
+(oracle with the kernel's kv block; max-abs <= 2e-2 + the row's rounding-flip allowance, mean-abs <= 2e-3)."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import cutlass_flash_atten_fp8_amd as fa
+from oracle import fa8_oracle as fo
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def draw_case(rng):
+    d = int(rng.choice([32, 64, 96, 128, 160, 192, 224, 256]))
+    hk = int(rng.choice([1, 2, 3]))
+    h = hk * int(rng.choice([1, 2, 4]))
+    b = int(rng.integers(1, 3))
+    nq = int(rng.choice([1, 7, 33, 64, 65, 127, 128, 129, 191, 200, 256, 300, 511, 640]))
+    causal = bool(rng.integers(0, 2))
+    nk = nq if rng.integers(0, 2) else int(rng.choice([1, 16, 48, 64, 80, 128, 144, 272, 400, 704]))
+    vt = bool(rng.integers(0, 2)) and nk % 16 == 0
+    e5m2 = bool(rng.integers(0, 4) == 0)
+    out8 = (not e5m2) and bool(rng.integers(0, 4) == 0)
+    return dict(b=b, h=h, hk=hk, nq=nq, nk=nk, d=d, causal=causal, bottom_right=bool(rng.integers(0, 2)), vt=vt, e5m2=e5m2,
+                out8=out8, scale=float(rng.choice([1.0, 0.5, 2.0])) / math.sqrt(d), spread=float(rng.choice([0.5, 1.0, 2.0])))
+
+
+CASES = [draw_case(np.random.default_rng(1000 + i)) for i in range(64)]
+
+
+@pytest.mark.parametrize("case", CASES, ids=[f"{i}" for i in range(len(CASES))])
+def test_random_case(case):
+    c = case
+    print(f"[random] {c}", flush=True)
+    in_dtype = torch.float8_e5m2 if c["e5m2"] else torch.float8_e4m3fn
+    g = torch.Generator().manual_seed(c["nq"] * 1000 + c["nk"] + c["d"])
+    q = (torch.randn((c["b"], c["h"], c["nq"], c["d"]), generator=g) * c["spread"]).to(in_dtype)
+    k = (torch.randn((c["b"], c["hk"], c["nk"], c["d"]), generator=g) * c["spread"]).to(in_dtype)
+    v = torch.randn((c["b"], c["hk"], c["nk"], c["d"]), generator=g).to(in_dtype)
+    v_arg = v.transpose(2, 3).contiguous() if c["vt"] else v
+    res = fa.flash_attention_v2_cutlass(q.to(DEV), k.to(DEV), v_arg.to(DEV), c["causal"], c["scale"], v_transposed=c["vt"],
+                                        out_dtype=torch.float8_e4m3fn if c["out8"] else None, return_lse=True,
+                                        causal_bottom_right=c["bottom_right"])
+    o, lse = res[0].float().cpu().numpy(), res[1].cpu().numpy()
+    u8 = [t.view(torch.uint8).numpy() for t in (q, k, v)]
+    ref, allow, ref_lse = fo.forward(*u8, c["scale"], causal=c["causal"], kv_block=fa.query(fa.FA8_QUERY_KV_BLOCK),
+                                     in_dtype=fo.E5M2 if c["e5m2"] else fo.E4M3, exp2_form=True, logit_rel_err=2e-5,
+                                     causal_bottom_right=c["bottom_right"], return_lse=True, out_dtype=fo.OUT_F32)
+    assert np.isfinite(o).all()
+    err = np.abs(o - ref)
+    # an e4m3 output adds its own rounding: half a step of the value (3 mantissa bits), at least half the smallest subnormal
+    out_round = np.maximum(np.abs(ref) * 2.0 ** -4, 2.0 ** -10).max(axis=-1) if c["out8"] else 0.0
+    assert (err.max(axis=-1) <= 2e-2 + allow + out_round).all(), float(err.max())
+    assert err.mean() <= (2e-3 if not c["out8"] else 2e-2)
+    empty = np.isneginf(ref_lse)
+    assert np.array_equal(np.isneginf(lse), empty)
+    if (~empty).any():
+        assert np.abs(lse[~empty] - ref_lse[~empty]).max() <= 5e-4 * max(1.0, np.abs(ref_lse[~empty]).max())
+    assert (o[empty] == 0).all()
