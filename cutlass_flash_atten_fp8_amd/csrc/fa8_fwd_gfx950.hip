@@ -470,7 +470,16 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
       compute_tile(j + 2, k_lds0, v_lds0, std::false_type());
       stage_sync(true);
     }
-    // The remaining blocks (the last few mask-free ones, the blocks on the diagonal, the kv tail) take the masking copy.
+    // The last few mask-free blocks: same arithmetic, LDS stage chosen at run time, copies issued while blocks remain.
+    for (; j < n_plain; ++j) {
+      const int st = j % 3, st2 = (j + 2) % 3;
+      if (j + 2 < n_tiles)
+        issue_tile(j + 2, st2 == 0 ? k_lds0 : (st2 == 1 ? k_lds1 : k_lds2), st2 == 0 ? v_lds0 : (st2 == 1 ? v_lds1 : v_lds2));
+      compute_tile(j, st == 0 ? k_lds0 : (st == 1 ? k_lds1 : k_lds2), st == 0 ? v_lds0 : (st == 1 ? v_lds1 : v_lds2),
+                   std::false_type());
+      stage_sync(j + 2 < n_tiles);
+    }
+    // The remaining blocks (the blocks on the diagonal, the kv tail) take the masking copy.
     for (; j < n_tiles; ++j) {
       const int st = j % 3, st2 = (j + 2) % 3;
       if (j + 2 < n_tiles)
@@ -495,6 +504,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
       stage_sync(false);
       issue_tile(j + 2, k_lds1, v_lds1);
       compute_tile(j + 1, k_lds0, v_lds0, std::false_type());
+      stage_sync(false);
+    }
+    for (; j < n_plain; ++j) {  // the last mask-free blocks
+      const bool odd = j & 1;
+      if (j + 1 < n_tiles) issue_tile(j + 1, odd ? k_lds0 : k_lds1, odd ? v_lds0 : v_lds1);
+      compute_tile(j, odd ? k_lds1 : k_lds0, odd ? v_lds1 : v_lds0, std::false_type());
       stage_sync(false);
     }
     for (; j < n_tiles; ++j) {
