@@ -169,6 +169,11 @@ typedef struct Fa8OracleArgs {
   int32_t heads_k;      /* k/v heads (0 = heads); q head h uses k/v head h / (heads / heads_k) */
   int32_t causal_shift; /* causal: column j is visible to row i when j <= i + causal_shift (reference: 0, :62-64) */
   float* lse;           /* optional float [B,H,n_rows]: scale*m + log(l) of the row, -inf when the row sees no column */
+  /* Second part of the logit error model behind flip_allow (0 = off): a matrix core that sums the products of
+   * trunc_group consecutive k indices after cutting each to 2^(e - trunc_bits), e the exponent of the largest product
+   * of the group (see logit_error_bound). */
+  int32_t trunc_group;
+  int32_t trunc_bits;
 } Fa8OracleArgs;
 
 /* number of leading columns row i sees */
@@ -208,10 +213,37 @@ static float dot_f32(const float* x, const float* y, int d) {
   return ((s[0] + s[1]) + (s[2] + s[3])) + ((s[4] + s[5]) + (s[6] + s[7]));
 }
 
-static float dot_abs_f32(const float* x, const float* y, int d) {
-  float s = 0.0f;
-  for (int i = 0; i < d; ++i) s += fabsf(x[i] * y[i]);
-  return s;
+/* Bound on |S_device - S_exact| for one logit S = sum_k x_k y_k under the error model of the arguments:
+ *   logit_rel_err * sum_k |x_k y_k|                      (accumulation that is not IEEE fp32, order unknown)
+ * + the truncation of a matrix core that aligns the products of each group of trunc_group consecutive k to the
+ *   largest product of the group and cuts them (toward zero) to the grid 2^(e_g - trunc_bits), e_g the exponent of
+ *   that largest product: every other non-zero product of the group loses up to one grid step.  The sum of those
+ *   losses is bounded by their worst case and, being independent cuts of terms of either sign, by four standard
+ *   deviations (a uniform cut has a second moment of step^2 / 3); the smaller of the two is taken. */
+static float logit_error_bound(const Fa8OracleArgs* a, const float* x, const float* y, int d) {
+  float sum_abs = 0.0f;
+  double worst = 0.0, var = 0.0;
+  const int g = a->trunc_group;
+  for (int k0 = 0; k0 < d; k0 += (g > 0 ? g : d)) {
+    const int k1 = (g > 0 && k0 + g < d) ? k0 + g : d;
+    float gmax = 0.0f;
+    int nz = 0;
+    for (int k = k0; k < k1; ++k) {
+      const float t = fabsf(x[k] * y[k]);
+      sum_abs += t;
+      if (t > gmax) gmax = t;
+      if (t > 0.0f) ++nz;
+    }
+    if (g > 0 && nz > 1) {
+      int e;
+      (void)frexpf(gmax, &e); /* gmax = f * 2^e, f in [0.5, 1): exponent of the leading bit is e - 1 */
+      const double step = ldexp(1.0, e - 1 - a->trunc_bits);
+      worst += (nz - 1) * step;
+      var += (nz - 1) * step * step / 3.0;
+    }
+  }
+  const double stat = 4.0 * sqrt(var);
+  return a->logit_rel_err * sum_abs + (float)(worst < stat ? worst : stat);
 }
 
 /* Relative distance of p (0 < p <= max) to the nearest point where its fp8 rounding changes, and the size of
@@ -235,13 +267,14 @@ static void oracle_row(const Fa8OracleArgs* a, const float* qrow, const float* k
    * from the exact ones by a few 1e-5 of sum|q_k k_k| (matrix cores do not accumulate in IEEE fp32) can round a
    * P that lies next to a rounding boundary the other way: a legitimate one-quantum difference that changes
    * O[i,:] by quantum * V[j,:] / l.  *flip_allow returns the sum of those possible changes (times max|V[j,:]|)
-   * over the columns whose P is within reach of a boundary given a->logit_rel_err. */
+   * over the columns whose P is within reach of a boundary given the logit error model (logit_error_bound). */
   const int d = a->head_dim, nk = a->seqlen_k, bc = a->kv_block;
   float allow = 0.0f;
   const int mbits = a->in_dtype == FA8O_E5M2 ? 2 : 3, emin = a->in_dtype == FA8O_E5M2 ? -14 : -6;
   const float scale = a->softmax_scale;
   const float c2 = scale * 1.4426950408889634f;
   float m = -INFINITY, l = 0.0f;
+  float m_bound = 0.0f; /* logit error bound of the column that holds the running max */
   for (int x = 0; x < d; ++x) acc[x] = 0.0f;
   /* Reference loop bound (:458): every block that starts before the end of the row's q block.  Blocks that
    * start after column i are fully masked for this row (m, l and O unchanged), so the loop may stop at j0 <= i. */
@@ -249,13 +282,18 @@ static void oracle_row(const Fa8OracleArgs* a, const float* qrow, const float* k
   for (int j0 = 0; j0 < j_end; j0 += bc) {
     const int jn = j0 + bc < nk ? j0 + bc : nk; /* the block covers columns [j0, jn) */
     float bmax = -INFINITY;
+    int jmax = -1;
     for (int j = j0; j < jn; ++j) {
       /* S = q . k_j in fp32 (:487); causal mask: column > row -> -inf (:62-64) */
       const float s = j < j_end ? dot_f32(qrow, kf + (size_t)j * d, d) : -INFINITY;
       p[j - j0] = s;
-      if (s > bmax) bmax = s;
+      if (s > bmax) {
+        bmax = s;
+        jmax = j;
+      }
     }
     const float m_new = m > bmax ? m : bmax; /* max over the raw logits (:238, :249) */
+    if (flip_allow && bmax > m && jmax >= 0) m_bound = logit_error_bound(a, qrow, kf + (size_t)jmax * d, d);
     if (m != -INFINITY) {                    /* not the first block: rescale l and O (:258-261) */
       const float alpha = a->exp2_form ? exp2f((m - m_new) * c2) : expf((m - m_new) * scale);
       l *= alpha;
@@ -271,8 +309,8 @@ static void oracle_row(const Fa8OracleArgs* a, const float* qrow, const float* k
       if (flip_allow && a->quantize_p && j < j_end && pj > 0.0f) {
         float quantum;
         const float dist = tie_distance(pj, mbits, emin, &quantum);
-        /* the device logit and the device row max may each be off by logit_rel_err * sum|terms| */
-        const float reach = 2.0f * fabsf(scale) * a->logit_rel_err * dot_abs_f32(qrow, kf + (size_t)j * d, d);
+        /* the device logit and the device row max may each be off by their error bound */
+        const float reach = fabsf(scale) * (logit_error_bound(a, qrow, kf + (size_t)j * d, d) + m_bound);
         if (dist <= reach) {
           float vmax = 0.0f;
           for (int x = 0; x < d; ++x) vmax = fmaxf(vmax, fabsf(vf[(size_t)j * d + x]));

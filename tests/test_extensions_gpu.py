@@ -28,7 +28,7 @@ def u8(t):
 
 def gate(o, lse, q, k, v, scale, causal, bottom_right=False, label=""):
     ref, allow, ref_lse = fo.forward(u8(q), u8(k), u8(v), scale, causal=causal, kv_block=fa.query(fa.FA8_QUERY_KV_BLOCK),
-                                     exp2_form=True, logit_rel_err=2e-5, causal_bottom_right=bottom_right, return_lse=True)
+                                     exp2_form=True, causal_bottom_right=bottom_right, return_lse=True, **fo.MFMA_F8F6F4_ERROR_MODEL)
     got = o.float().cpu().numpy()
     assert np.isfinite(got).all()
     err = np.abs(got - ref.astype(np.float32))

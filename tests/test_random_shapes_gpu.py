@@ -48,7 +48,7 @@ def test_random_case(case):
     o, lse = res[0].float().cpu().numpy(), res[1].cpu().numpy()
     u8 = [t.view(torch.uint8).numpy() for t in (q, k, v)]
     ref, allow, ref_lse = fo.forward(*u8, c["scale"], causal=c["causal"], kv_block=fa.query(fa.FA8_QUERY_KV_BLOCK),
-                                     in_dtype=fo.E5M2 if c["e5m2"] else fo.E4M3, exp2_form=True, logit_rel_err=2e-5,
+                                     in_dtype=fo.E5M2 if c["e5m2"] else fo.E4M3, exp2_form=True, **fo.MFMA_F8F6F4_ERROR_MODEL,
                                      causal_bottom_right=c["bottom_right"], return_lse=True, out_dtype=fo.OUT_F32)
     assert np.isfinite(o).all()
     err = np.abs(o - ref)
