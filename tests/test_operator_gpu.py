@@ -206,3 +206,29 @@ def test_error_paths_raise_and_launch_nothing():
     o = ext.flash_attention_v2_cutlass(q, k_short, k_short, False, 0.1)[0]
     ref = fo.forward(u8(q), u8(k_short), u8(k_short), 0.1, exp2_form=True).astype(np.float32)
     assert np.abs(o.float().cpu().numpy() - ref).mean() <= 2e-3
+
+
+def test_capturable_in_a_hip_graph():
+    """The launcher allocates nothing and never synchronises, so the operator can be recorded into a HIP graph
+    (here through torch.cuda.graph, whose allocator provides the output inside the capture) and replayed."""
+    ext = fa.load_extension()
+    q, k, v = (rand_fp8((2, 4, 384, 128), s).to(DEV) for s in (50, 51, 52))
+    eager = ext.flash_attention_v2_cutlass(q, k, v, True, 0.09)[0].clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):  # warm-up outside the capture, as torch asks
+        ext.flash_attention_v2_cutlass(q, k, v, True, 0.09)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = ext.flash_attention_v2_cutlass(q, k, v, True, 0.09)[0]
+    for i in range(3):
+        out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), f"replay {i}"
+        # eager work and new inputs between replays: the graph reads q/k/v in place
+        q.copy_(rand_fp8((2, 4, 384, 128), 60 + i).to(DEV))
+        eager = ext.flash_attention_v2_cutlass(q, k, v, True, 0.09)[0].clone()
