@@ -62,6 +62,23 @@ def reference_sweep(ext, torch):
                       "inputs N(0,0.5) clamped to +-0.1 (reference test.py:13-23,56-57)", "rows": rows}), flush=True)
 
 
+def read_sclk_mhz():
+    """Current shader clock from the amdgpu sysfs node (the level marked '*' in pp_dpm_sclk), or None."""
+    import glob
+    import re
+    for path in sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk")):
+        try:
+            with open(path) as f:
+                for line in f:
+                    if line.rstrip().endswith("*"):
+                        m = re.search(r"(\d+)\s*Mhz", line, re.IGNORECASE)
+                        if m:
+                            return int(m.group(1))
+        except OSError:
+            pass
+    return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -130,6 +147,17 @@ def main():
         e1.record()
     torch.cuda.synchronize()
     kern_ms = sorted(e0.elapsed_time(e1) for e0, e1 in evs)
+    # shader clock while the kernel is running (power management lowers it under dense matrix work): sampled in the
+    # middle of an untimed burst of launches, median of 16 readings
+    samples = []
+    for _ in range(20):
+        for _ in range(max(1, args.steps // 8)):
+            step()
+        time.sleep(0.004)  # the queue stays full: the launches above take longer than this
+        samples.append(read_sclk_mhz())
+    torch.cuda.synchronize()
+    samples = sorted(x for x in samples[4:] if x is not None)
+    sclk = samples[len(samples) // 2] if samples else None
     kern_avg_ms = sum(kern_ms) / len(kern_ms)
 
     tflops = flops / (wall_ms * 1e-3) / 1e12
@@ -156,6 +184,7 @@ def main():
             "pct_fp8_mfma_peak": round(100.0 * tflops / FP8_MFMA_PEAK_TFLOPS, 2),
             "algorithmic_hbm_gbps": round(alg_bytes / (kern_avg_ms * 1e-3) / 1e9, 1),
             "kv_block": fa.query(fa.FA8_QUERY_KV_BLOCK),
+            "sclk_mhz_under_load": sclk,
         },
         "roofline": {
             "bound": "mfma",
