@@ -14,7 +14,10 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "liboracle.so")
 
 E4M3, E5M2 = 0, 1
-OUT_FP16, OUT_E4M3, OUT_F32 = 0, 1, 2
+OUT_FP16, OUT_E4M3, OUT_F32, OUT_E5M2 = 0, 1, 2, 3
+# how the two matrix products are summed: IEEE fp32 in a fixed order, or as the gfx950 instruction
+# v_mfma_f32_32x32x64_f8f6f4 does (fa8o_mfma_32x32x64_f8 in fa8_oracle.c, pinned by recorded hardware vectors)
+MATMUL_IEEE, MATMUL_GFX950 = 0, 1
 
 
 class _Args(ctypes.Structure):
@@ -26,7 +29,7 @@ class _Args(ctypes.Structure):
         ("v_transposed", ctypes.c_int32), ("quantize_p", ctypes.c_int32), ("exp2_form", ctypes.c_int32),
         ("softmax_scale", ctypes.c_float), ("flip_allow", ctypes.c_void_p), ("logit_rel_err", ctypes.c_float),
         ("heads_k", ctypes.c_int32), ("causal_shift", ctypes.c_int32), ("lse", ctypes.c_void_p),
-        ("trunc_group", ctypes.c_int32), ("trunc_bits", ctypes.c_int32),
+        ("trunc_group", ctypes.c_int32), ("trunc_bits", ctypes.c_int32), ("matmul_model", ctypes.c_int32),
     ]
 
 
@@ -70,6 +73,8 @@ def lib():
         L.fa8o_attention_f64.restype = ctypes.c_int
         L.fa8o_attention_f64.argtypes = [ctypes.POINTER(_Args), ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p]
         L.fa8o_num_threads.restype = ctypes.c_int
+        L.fa8o_mfma_32x32x64_f8.restype = ctypes.c_float
+        L.fa8o_mfma_32x32x64_f8.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_float, ctypes.c_int]
         _lib = L
     return _lib
 
@@ -88,10 +93,12 @@ def _prep(q, k, v, v_transposed):
 
 def forward(q, k, v, scale, causal=False, kv_block=64, rows=None, in_dtype=E4M3, out_dtype=OUT_FP16,
             v_transposed=False, quantize_p=True, exp2_form=False, logit_rel_err=None, causal_bottom_right=False,
-            return_lse=False, trunc_group=0, trunc_bits=0):
+            return_lse=False, trunc_group=0, trunc_bits=0, matmul_model=MATMUL_IEEE):
     """The reference pipeline on uint8 views of fp8 q/k/v [B,H,N,d].
 
-    Returns [B,H,n_rows,d] as float16 (OUT_FP16), uint8 e4m3 codes (OUT_E4M3) or float32 (OUT_F32).
+    Returns [B,H,n_rows,d] as float16 (OUT_FP16), uint8 fp8 codes (OUT_E4M3, OUT_E5M2) or float32 (OUT_F32).
+    matmul_model: MATMUL_IEEE sums both products in fp32; MATMUL_GFX950 sums them as the MI355X matrix instruction
+    does (needs kv_block 64 and a head dim that is a multiple of 32).
     rows: optional 1-D int array of query rows to evaluate for every (batch, head).
     logit_rel_err: when given, also returns flip_allow float32 [B,H,n_rows]: how much O[row,:] may legitimately
     move because some P sits within reach of an fp8 rounding boundary for a device whose logits are accurate
@@ -105,7 +112,7 @@ def forward(q, k, v, scale, causal=False, kv_block=64, rows=None, in_dtype=E4M3,
     q, k, v, B, H, nq, nk, d, hk = _prep(q, k, v, v_transposed)
     rows_arr = None if rows is None else np.ascontiguousarray(rows, dtype=np.int32)
     nr = nq if rows_arr is None else int(rows_arr.shape[0])
-    np_dtype = {OUT_FP16: np.uint16, OUT_E4M3: np.uint8, OUT_F32: np.float32}[out_dtype]
+    np_dtype = {OUT_FP16: np.uint16, OUT_E4M3: np.uint8, OUT_E5M2: np.uint8, OUT_F32: np.float32}[out_dtype]
     o = np.zeros((B, H, nr, d), dtype=np_dtype)
     allow = None if logit_rel_err is None else np.zeros((B, H, nr), dtype=np.float32)
     lse = np.zeros((B, H, nr), dtype=np.float32) if return_lse else None
@@ -113,7 +120,7 @@ def forward(q, k, v, scale, causal=False, kv_block=64, rows=None, in_dtype=E4M3,
               int(kv_block), int(in_dtype), int(out_dtype), int(bool(v_transposed)), int(bool(quantize_p)),
               int(bool(exp2_form)), float(scale), None if allow is None else allow.ctypes.data,
               0.0 if logit_rel_err is None else float(logit_rel_err), hk, nk - nq if causal_bottom_right else 0,
-              None if lse is None else lse.ctypes.data, int(trunc_group), int(trunc_bits))
+              None if lse is None else lse.ctypes.data, int(trunc_group), int(trunc_bits), int(matmul_model))
     rc = lib().fa8o_fwd_rows(ctypes.byref(a), None if rows_arr is None else rows_arr.ctypes.data, nr)
     if rc != 0:
         raise RuntimeError(f"fa8o_fwd_rows failed with {rc}")
@@ -130,12 +137,21 @@ def attention_f64(q, k, v, scale, causal=False, rows=None, in_dtype=E4M3, v_tran
     o = np.zeros((B, H, nr, d), dtype=np.float64)
     a = _Args(q.ctypes.data, k.ctypes.data, v.ctypes.data, None, B, H, nq, nk, d, int(bool(causal)), 64,
               int(in_dtype), OUT_F32, int(bool(v_transposed)), 0, 0, float(scale), None, 0.0, hk,
-              nk - nq if causal_bottom_right else 0, None, 0, 0)
+              nk - nq if causal_bottom_right else 0, None, 0, 0, 0)
     rc = lib().fa8o_attention_f64(ctypes.byref(a), None if rows_arr is None else rows_arr.ctypes.data, nr,
                                   o.ctypes.data)
     if rc != 0:
         raise RuntimeError(f"fa8o_attention_f64 failed with {rc}")
     return o
+
+
+def mfma_32x32x64(x, y, c=0.0, fmt=E4M3):
+    """One output element of v_mfma_f32_32x32x64_f8f6f4 as the oracle models it: x, y 64 fp8 codes (uint8), c the
+    accumulator input; returns float32."""
+    x = np.ascontiguousarray(x, dtype=np.uint8)
+    y = np.ascontiguousarray(y, dtype=np.uint8)
+    assert x.shape == (64,) and y.shape == (64,)
+    return np.float32(lib().fa8o_mfma_32x32x64_f8(x.ctypes.data, y.ctypes.data, float(np.float32(c)), int(fmt)))
 
 
 def num_threads():

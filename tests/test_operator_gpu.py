@@ -9,6 +9,7 @@ import torch
 
 import cutlass_flash_atten_fp8_amd as fa
 from oracle import fa8_oracle as fo
+from oracle.parity_gate import assert_parity
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -154,11 +155,7 @@ def test_e5m2_inputs_match_oracle(causal, d):
     q, k, v = (rand_fp8((2, 2, 333, d), s, dtype=torch.float8_e5m2) for s in (27, 28, 29))
     scale = 1 / math.sqrt(d)
     o = fa.flash_attention_v2_cutlass(q.to(DEV), k.to(DEV), v.to(DEV), causal, scale)[0].float().cpu().numpy()
-    ref, allow = fo.forward(u8(q), u8(k), u8(v), scale, causal=causal, exp2_form=True, in_dtype=fo.E5M2, **fo.MFMA_F8F6F4_ERROR_MODEL)
-    err = np.abs(o - ref.astype(np.float32))
-    print(f"e5m2 d={d} causal={causal}: max {err.max():.3e} mean {err.mean():.3e}")
-    assert (err.max(axis=-1) <= 2e-2 + allow).all()
-    assert err.mean() <= 2e-3
+    assert_parity(o, u8(q), u8(k), u8(v), scale, causal=causal, in_dtype=fo.E5M2, label=f"e5m2 d={d} causal={causal}")
 
 
 @pytest.mark.parametrize("causal", [False, True])
@@ -174,8 +171,8 @@ def test_transposed_v_is_the_reference_calling_convention(n, d, causal):
     ot = ext.flash_attention_v2_cutlass(q, k, vt, causal, 0.1, v_transposed=True)[0]
     torch.cuda.synchronize()
     assert torch.equal(o, ot)
-    ref = fo.forward(u8(q.cpu()), u8(k.cpu()), u8(vt.cpu()), 0.1, causal=causal, exp2_form=True, v_transposed=True)
-    assert np.abs(ot.float().cpu().numpy() - ref.astype(np.float32)).mean() <= 2e-3
+    assert_parity(ot.float().cpu().numpy(), u8(q), u8(k), u8(vt), 0.1, causal=causal, v_transposed=True,
+                  label=f"transposed v n={n} d={d} causal={causal}")
 
 
 def test_error_paths_raise_and_launch_nothing():
