@@ -27,6 +27,9 @@ MEASURED_TRAFFIC_BYTES = {"cfg3": 168.0e6,  # profiles/fa8_fwd_kernel_d128_cfg3_
                           "cfg2": 21.2e6, "cfg4": 173.2e6, "cfg5": 103.1e6}  # profiles/fa8_fwd_kernel_cfg2_cfg4_cfg5.md
 
 
+TRAFFIC_SOURCE = {"cfg3": "profiles/fa8_fwd_kernel_d128_cfg3_headline.md", "cfg2": "profiles/fa8_fwd_kernel_cfg2_cfg4_cfg5.md",
+                  "cfg4": "profiles/fa8_fwd_kernel_cfg2_cfg4_cfg5.md", "cfg5": "profiles/fa8_fwd_kernel_cfg2_cfg4_cfg5.md"}
+
 # cutlass fp8 milliseconds published by the reference (benchmark.png, rows in the order of test.py:95-100; Ada sm_89,
 # GPU model unstated; host wall clock with a device sync per iteration)
 REFERENCE_MS = {(16, 1024, 64): 0.0352, (16, 1024, 128): 0.0500, (16, 2048, 64): 0.0833, (16, 2048, 128): 0.1169,
@@ -86,6 +89,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="cfg3", help="cfg1..cfg5 (cfg3 is the headline)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--settle-seconds", type=float, default=0.25,
+                    help="untimed launches for this long after the warm-up, so that the shader clock has settled")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the baseline sample")
     ap.add_argument("--reference-sweep", action="store_true",
                     help="instead of the headline step, time the 18 shapes of the reference's own benchmark table "
@@ -132,6 +137,15 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
+    # Clock settle (untimed, disclosed as config.settle_launches): after an idle period the first launches run at a
+    # lower shader clock, whatever --warmup says; keep the GPU busy for a fixed time before anything is timed.
+    settle_launches = 0
+    t_settle = time.perf_counter()
+    while time.perf_counter() - t_settle < args.settle_seconds:
+        for _ in range(50):
+            step()
+        torch.cuda.synchronize()
+        settle_launches += 50
     # whole-step wall clock: exactly `steps` steps between two device synchronisations
     t0 = time.perf_counter()
     for _ in range(args.steps):
@@ -148,12 +162,13 @@ def main():
     torch.cuda.synchronize()
     kern_ms = sorted(e0.elapsed_time(e1) for e0, e1 in evs)
     # shader clock while the kernel is running (power management lowers it under dense matrix work): sampled in the
-    # middle of an untimed burst of launches, median of 16 readings
+    # middle of untimed bursts of launches long enough to keep the queue full whatever --steps is, median of 16 readings
+    burst = max(25, int(0.008 / max(kern_ms[len(kern_ms) // 2] * 1e-3, 1e-6)))  # about 8 ms of kernel time per burst
     samples = []
     for _ in range(20):
-        for _ in range(max(1, args.steps // 8)):
+        for _ in range(burst):
             step()
-        time.sleep(0.004)  # the queue stays full: the launches above take longer than this
+        time.sleep(0.004)  # the queue stays full: the launches above take about twice as long as this
         samples.append(read_sclk_mhz())
     torch.cuda.synchronize()
     samples = sorted(x for x in samples[4:] if x is not None)
@@ -185,6 +200,7 @@ def main():
             "algorithmic_hbm_gbps": round(alg_bytes / (kern_avg_ms * 1e-3) / 1e9, 1),
             "kv_block": fa.query(fa.FA8_QUERY_KV_BLOCK),
             "sclk_mhz_under_load": sclk,
+            "settle_launches": settle_launches,
         },
         "roofline": {
             "bound": "mfma",
@@ -193,6 +209,8 @@ def main():
             "unit": "TFLOP/s",
             "frac": round(kern_tflops / FP8_MFMA_PEAK_TFLOPS, 4),
             "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+            "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a plain copy: " + TRAFFIC_SOURCE[args.workload]
+                              if args.workload in TRAFFIC_SOURCE else None,
             "kernel_ms_avg": round(kern_avg_ms, 5),
             "kernel_ms_min": round(kern_ms[0], 5),
             "kernel_ms_median": round(kern_ms[len(kern_ms) // 2], 5),
@@ -203,8 +221,8 @@ def main():
         # The reference's CPU-runnable path (naive attention, reference test.py:25-33) restated in oracle/ and timed
         # on this machine's host cores, on the first heads of the same workload.
         from oracle.naive_attention import naive_attention_cpu
-        cores = os.cpu_count() or 1
-        threads = min(cores, 16)
+        host_cores = os.cpu_count() or 1
+        threads = min(host_cores, 16)  # a one-GPU box shares its host: 16 cores are this job's share
         torch.set_num_threads(threads)
         naive_attention_cpu(q8, k8, v8, scale, causal, heads_limit=1)  # warm-up, also sizes the sample
         t0 = time.perf_counter()
@@ -221,7 +239,8 @@ def main():
         out["cpu_baseline"] = {
             "value": round(cpu_tflops, 4),
             "unit": "TFLOP/s",
-            "cores": threads,
+            "cores": threads,  # threads actually used
+            "host_cores": host_cores,  # os.cpu_count() of the machine
             "kind": "port",
             "sample": f"first {n} of {n_heads_total} (batch*head) slices of the same workload, {reps} pass(es) of "
                       f"{cpu_s:.2f} s, torch CPU naive attention with P re-quantised to e4m3",

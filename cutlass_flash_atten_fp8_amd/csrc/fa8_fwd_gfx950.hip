@@ -126,8 +126,11 @@ __device__ __forceinline__ void tile_slot_decode(int slot, int& row, int& chunk)
 typedef unsigned v2u __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ float lane32_max(float x) {
   const v2u r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-  // median(a, b, +inf) = max(a, b) in one instruction (fmaxf would first quiet both operands)
-  return __builtin_amdgcn_fmed3f(__uint_as_float(r[0]), __uint_as_float(r[1]), INFINITY);
+  // median(a, b, +inf) = max(a, b) in one instruction (fmaxf would first quiet both operands); the +inf is made opaque to
+  // the optimiser, which would otherwise turn the median back into that max
+  float inf = INFINITY;
+  asm("" : "+v"(inf));
+  return __builtin_amdgcn_fmed3f(__uint_as_float(r[0]), __uint_as_float(r[1]), inf);
 }
 __device__ __forceinline__ float lane32_sum(float x) {
   const v2u r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
@@ -364,12 +367,16 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
           if (kv0 + 32 * h + 16 * t + i > kv_limit) s[t][i] = -INFINITY;
     }
     // ---- online softmax (reference softmax_rescale_o, csrc/flash_attention.cu:233-273) ----
-    float mx[4] = {m_run, m_run, m_run, m_run};  // four independent chains; sub-tile 0 first (it is ready first)
+    // 33 values (32 logits and the running max) in 16 three-input maxima: four independent chains over sub-tile 0
+    // (it is ready first), then sub-tile 1
+    float mx[4];
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+    for (int ch = 0; ch < 4; ++ch) mx[ch] = max3(s[0][4 * ch], s[0][4 * ch + 1], s[0][4 * ch + 2]);
 #pragma unroll
-      for (int i = 0; i < 16; i += 2) mx[(i >> 1) & 3] = max3(mx[(i >> 1) & 3], s[t][i], s[t][i + 1]);
-    const float m_new = lane32_max(max3(max3(mx[0], mx[1], mx[2]), mx[3], mx[3]));  // same in both half-lanes
+    for (int ch = 0; ch < 4; ++ch) mx[ch] = max3(mx[ch], s[0][4 * ch + 3], s[1][4 * ch]);
+#pragma unroll
+    for (int ch = 0; ch < 4; ++ch) mx[ch] = max3(mx[ch], s[1][4 * ch + 1], s[1][4 * ch + 2]);
+    const float m_new = lane32_max(max3(max3(mx[0], s[1][3], s[1][7]), max3(mx[1], s[1][11], s[1][15]), max3(mx[2], mx[3], m_run)));
     if (__any(m_new != m_run)) {
       float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * c);
       if constexpr (kMasked) alpha = (m_run == -INFINITY) ? 0.f : alpha;
@@ -382,7 +389,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
     }
     float mc = m_new * c;
     if constexpr (kMasked) mc = (m_new == -INFINITY) ? 0.f : mc;
-    float sum0 = 0.f, sum1 = 0.f;
+    float sum0, sum1;  // row sum of this block in two chains, started from the first two weights
     v8i p8;
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
@@ -396,8 +403,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
       }
 #pragma unroll
       for (int i = 0; i < 16; i += 2) {
-        sum0 += s[t][i];
-        sum1 += s[t][i + 1];
+        sum0 = (t == 0 && i == 0) ? s[t][i] : sum0 + s[t][i];
+        sum1 = (t == 0 && i == 0) ? s[t][i + 1] : sum1 + s[t][i + 1];
       }
 #pragma unroll
       for (int w = 0; w < 4; ++w)
