@@ -23,7 +23,7 @@ EXT_PATH = os.path.join(_PKG_DIR, _EXT_NAME + sysconfig.get_config_var("EXT_SUFF
 
 # codes of include/fa8_api.h
 FA8_DTYPE_E4M3, FA8_DTYPE_E5M2 = 0, 1
-FA8_OUT_FP16, FA8_OUT_E4M3 = 0, 1
+FA8_OUT_FP16, FA8_OUT_E4M3, FA8_OUT_E5M2 = 0, 1, 2
 FA8_V_ROWS, FA8_V_TRANSPOSED = 0, 1
 FA8_CAUSAL_TOP_LEFT, FA8_CAUSAL_BOTTOM_RIGHT = 0, 1
 (FA8_QUERY_VERSION, FA8_QUERY_KV_BLOCK, FA8_QUERY_Q_BLOCK, FA8_QUERY_KV_ASCENDING, FA8_QUERY_THREADS,
@@ -99,13 +99,13 @@ def make_params(q, k, v, o, is_causal, softmax_scale, v_transposed=False, lse=No
     k and v may have fewer heads than q (grouped-query attention); lse, if given, is a float32 [B,H,Nq] output."""
     import torch
     in_codes = {torch.float8_e4m3fn: FA8_DTYPE_E4M3, torch.float8_e5m2: FA8_DTYPE_E5M2}
-    out_codes = {torch.float16: FA8_OUT_FP16, torch.float8_e4m3fn: FA8_OUT_E4M3}
+    out_codes = {torch.float16: FA8_OUT_FP16, torch.float8_e4m3fn: FA8_OUT_E4M3, torch.float8_e5m2: FA8_OUT_E5M2}
     if q.dtype not in in_codes:
         raise RuntimeError(f"q must be torch.float8_e4m3fn or torch.float8_e5m2 (OCP fp8), got {q.dtype}")
     if k.dtype != q.dtype or v.dtype != q.dtype:
         raise RuntimeError("q, k and v must have the same dtype")
     if o.dtype not in out_codes:
-        raise RuntimeError("out_dtype must be torch.float16 or torch.float8_e4m3fn")
+        raise RuntimeError("out_dtype must be torch.float16 or the fp8 type of the inputs")
     for name, t in (("q", q), ("k", k), ("v", v), ("o", o)):
         if t.dim() != 4:
             raise RuntimeError(f"{name} must be 4-dimensional [batch, heads, seqlen, head_dim], got {t.dim()} dims")
@@ -138,8 +138,8 @@ def flash_attention_v2_cutlass(q, k, v, is_causal, softmax_scale, *, v_transpose
     """The reference operator (reference csrc/flash_attention.cu:639-668) through the C ABI.
 
     q, k: fp8 [B,H,N,d] on the GPU; v: [B,H,N,d] (or [B,H,d,N] with v_transposed=True, as the reference
-    requires of its caller, test.py:71).  Returns [O], O fp16 [B,H,N,d] (out_dtype=torch.float8_e4m3fn
-    gives the reference's fp8 O).  Runs on torch's current stream without synchronising.  Raises
+    requires of its caller, test.py:71).  Returns [O], O fp16 [B,H,N,d] (out_dtype=q.dtype gives the
+    reference's fp8 O, stored in the input element type).  Runs on torch's current stream without synchronising.  Raises
     RuntimeError on bad arguments, like the reference's TORCH_CHECKs (include/attention_api.cuh:12-18).
     Beyond the reference: k/v may have fewer heads than q (grouped-query attention), return_lse=True returns
     [O, lse] with lse the float32 [B,H,Nq] log-sum-exp of the scaled logits, causal_bottom_right=True aligns the

@@ -7,7 +7,7 @@
 //
 // Deliberate differences from the reference host code:
 //   * v is [B,H,N,d] like k by default; `v_transposed=True` takes the reference's [B,H,d,N] (test.py:71);
-//   * O is fp16 by default; `out_dtype=torch.float8_e4m3fn` gives the reference's fp8 O (:656);
+//   * O is fp16 by default; `out_dtype=q.dtype` gives the reference's fp8 O in the input element type (:557, :656);
 //   * the kernel runs on torch's current stream and the call does not synchronise the device (:661-665);
 //   * bad arguments and HIP errors raise RuntimeError instead of printf + exit (include/attention_api.cuh:20-29).
 // Additions the reference declares but never implements (csrc/flash.h:36-45,56): k/v may have fewer heads than q
@@ -58,7 +58,8 @@ std::vector<torch::Tensor> flash_attention_v2_cutlass(torch::Tensor q, torch::Te
   TORCH_CHECK(B >= 1 && H >= 1 && Nq >= 1 && Nk >= 1, "empty tensors are not supported");
   TORCH_CHECK(Nq <= INT32_MAX && Nk <= INT32_MAX && B <= INT32_MAX && H <= INT32_MAX, "tensor too large");
   const at::ScalarType o_type = out_dtype.value_or(at::kHalf);
-  TORCH_CHECK(o_type == at::kHalf || o_type == at::kFloat8_e4m3fn, "out_dtype must be torch.float16 or torch.float8_e4m3fn");
+  TORCH_CHECK(o_type == at::kHalf || o_type == in_type,
+              "out_dtype must be torch.float16 or the fp8 type of the inputs (the reference's output type), got ", o_type);
 
   auto out = torch::empty({B, H, Nq, D}, q.options().dtype(o_type));
   torch::Tensor lse;
@@ -76,7 +77,7 @@ std::vector<torch::Tensor> flash_attention_v2_cutlass(torch::Tensor q, torch::Te
   p.head_dim = (int32_t)D;
   p.is_causal = is_causal ? 1 : 0;
   p.in_dtype = in_type == at::kFloat8_e5m2 ? FA8_DTYPE_E5M2 : FA8_DTYPE_E4M3;
-  p.out_dtype = o_type == at::kHalf ? FA8_OUT_FP16 : FA8_OUT_E4M3;
+  p.out_dtype = o_type == at::kHalf ? FA8_OUT_FP16 : (o_type == at::kFloat8_e5m2 ? FA8_OUT_E5M2 : FA8_OUT_E4M3);
   p.v_layout = v_transposed ? FA8_V_TRANSPOSED : FA8_V_ROWS;
   p.softmax_scale = softmax_scale;
   p.q_batch_stride = q.stride(0); p.q_head_stride = q.stride(1); p.q_row_stride = q.stride(2);

@@ -557,12 +557,13 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
 #pragma unroll
         for (int a2 = 0; a2 < 4; ++a2) {
           float x[4];
+          constexpr float kMaxFinite = OUT == FA8_OUT_E5M2 ? 57344.f : 448.f;
 #pragma unroll
           for (int b2 = 0; b2 < 4; ++b2) {
             const float y = o_acc[mt][4 * a2 + b2] * inv;
-            x[b2] = (y != y) ? y : fminf(fmaxf(y, -448.f), 448.f);  // saturate to finite, keep NaN
+            x[b2] = (y != y) ? y : fminf(fmaxf(y, -kMaxFinite), kMaxFinite);  // saturate to finite, keep NaN
           }
-          *(int*)(op + 32 * mt + 8 * a2) = pack4_fp8<false>(x[0], x[1], x[2], x[3]);
+          *(int*)(op + 32 * mt + 8 * a2) = pack4_fp8<OUT == FA8_OUT_E5M2>(x[0], x[1], x[2], x[3]);
         }
     }
   }
@@ -572,11 +573,13 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
 template <int D, bool CAUSAL, bool E5M2, int OUT>
 int launch(const KernelArgs& a, bool v_transposed, hipStream_t stream) {
   const dim3 grid((unsigned)(a.bh_total * a.n_qblocks));
-  if (v_transposed)
-    hipLaunchKernelGGL((fa8_fwd_kernel<D, CAUSAL, E5M2, OUT, true>), grid, dim3(kThreads), 0, stream, a);
-  else
-    hipLaunchKernelGGL((fa8_fwd_kernel<D, CAUSAL, E5M2, OUT, false>), grid, dim3(kThreads), 0, stream, a);
-  return (int)hipGetLastError();
+  // hipLaunchKernel returns the status of this launch itself; the thread's sticky "last error" (which an earlier,
+  // unrelated call may have left behind) is neither read nor cleared.
+  KernelArgs args = a;
+  void* argv[] = {&args};
+  const void* fn = v_transposed ? (const void*)&fa8_fwd_kernel<D, CAUSAL, E5M2, OUT, true>
+                                : (const void*)&fa8_fwd_kernel<D, CAUSAL, E5M2, OUT, false>;
+  return (int)hipLaunchKernel(fn, grid, dim3(kThreads), argv, 0, stream);
 }
 
 template <int D, bool CAUSAL>
@@ -584,9 +587,10 @@ int launch_types(const Fa8FwdParams* p, const KernelArgs& a, hipStream_t stream)
   const bool e5m2 = p->in_dtype == FA8_DTYPE_E5M2, vt = p->v_layout == FA8_V_TRANSPOSED;
   if (p->out_dtype == FA8_OUT_FP16)
     return e5m2 ? launch<D, CAUSAL, true, FA8_OUT_FP16>(a, vt, stream) : launch<D, CAUSAL, false, FA8_OUT_FP16>(a, vt, stream);
-  // fp8 output: the reference stores O in the input element type; only e4m3 out of e4m3 in is built
-  if (e5m2) return FA8_ERR_UNSUPPORTED;
-  return launch<D, CAUSAL, false, FA8_OUT_E4M3>(a, vt, stream);
+  // fp8 output: the reference stores O in the input element type (csrc/flash_attention.cu:557, :655-656); the two
+  // mixed combinations are not built
+  if (e5m2) return p->out_dtype == FA8_OUT_E5M2 ? launch<D, CAUSAL, true, FA8_OUT_E5M2>(a, vt, stream) : FA8_ERR_UNSUPPORTED;
+  return p->out_dtype == FA8_OUT_E4M3 ? launch<D, CAUSAL, false, FA8_OUT_E4M3>(a, vt, stream) : FA8_ERR_UNSUPPORTED;
 }
 
 bool span_ok(long long outer_stride, long long inner_extent) { return outer_stride >= inner_extent; }
@@ -601,7 +605,7 @@ extern "C" int fa8_fwd_validate(const Fa8FwdParams* p) {
   if (p->causal_align != FA8_CAUSAL_TOP_LEFT && p->causal_align != FA8_CAUSAL_BOTTOM_RIGHT) return FA8_ERR_DTYPE;
   if ((long long)p->batch * p->heads > 0x7fffffffLL / ((p->seqlen_q + kQBlock - 1) / kQBlock)) return FA8_ERR_SHAPE;
   if (p->in_dtype != FA8_DTYPE_E4M3 && p->in_dtype != FA8_DTYPE_E5M2) return FA8_ERR_DTYPE;
-  if (p->out_dtype != FA8_OUT_FP16 && p->out_dtype != FA8_OUT_E4M3) return FA8_ERR_DTYPE;
+  if (p->out_dtype != FA8_OUT_FP16 && p->out_dtype != FA8_OUT_E4M3 && p->out_dtype != FA8_OUT_E5M2) return FA8_ERR_DTYPE;
   if (p->v_layout != FA8_V_ROWS && p->v_layout != FA8_V_TRANSPOSED) return FA8_ERR_DTYPE;
   if (p->head_dim % 32 != 0 || p->head_dim > 256) return FA8_ERR_HEAD_DIM;
   if (!(p->softmax_scale == p->softmax_scale) || std::isinf(p->softmax_scale)) return FA8_ERR_SCALE;
@@ -627,11 +631,16 @@ extern "C" int fa8_fwd_validate(const Fa8FwdParams* p) {
     if (!span_ok(p->lse_head_stride, p->seqlen_q) || !span_ok(p->lse_batch_stride, 1)) return FA8_ERR_STRIDE;
     if ((uintptr_t)p->lse % 4 != 0) return FA8_ERR_ALIGN;
   }
-  // the kernels address k and v of one head with 32-bit byte offsets
-  if ((long long)p->seqlen_k * p->k_row_stride > 0x7fffffffLL || v_rows * p->v_row_stride > 0x7fffffffLL) return FA8_ERR_SHAPE;
+  // the kernels address k and v of one head with 32-bit byte offsets; a tile copy forms offsets for all 64 rows of a
+  // block (rows past the end are not read, but their offsets are computed), hence at least 64 rows here
+  const long long k_rows_addr = p->seqlen_k > kKvBlock ? p->seqlen_k : kKvBlock;
+  const long long v_rows_addr = v_rows > kKvBlock ? v_rows : kKvBlock;
+  if (k_rows_addr * p->k_row_stride > 0x7fffffffLL || v_rows_addr * p->v_row_stride > 0x7fffffffLL) return FA8_ERR_SHAPE;
   // transposed v is read in 16-byte chunks along kv
   if (p->v_layout == FA8_V_TRANSPOSED && p->seqlen_k % 16 != 0) return FA8_ERR_ALIGN;
-  if (p->in_dtype == FA8_DTYPE_E5M2 && p->out_dtype == FA8_OUT_E4M3) return FA8_ERR_UNSUPPORTED;
+  // an fp8 output has the element type of the inputs
+  if ((p->out_dtype == FA8_OUT_E4M3 && p->in_dtype != FA8_DTYPE_E4M3) || (p->out_dtype == FA8_OUT_E5M2 && p->in_dtype != FA8_DTYPE_E5M2))
+    return FA8_ERR_UNSUPPORTED;
   return FA8_OK;
 }
 
@@ -690,7 +699,7 @@ extern "C" const char* fa8_error_string(int code) {
   switch (code) {
     case FA8_OK: return "ok";
     case FA8_ERR_NULL: return "a required pointer is NULL";
-    case FA8_ERR_SHAPE: return "bad shape (a size < 1, too many workgroups, or heads not a multiple of heads_k)";
+    case FA8_ERR_SHAPE: return "bad shape (a size < 1, too many workgroups, heads not a multiple of heads_k, or k/v of one head spanning 2 GiB or more)";
     case FA8_ERR_HEAD_DIM: return "head_dim must be a multiple of 32, at most 256";
     case FA8_ERR_STRIDE: return "a stride is smaller than the extent it spans";
     case FA8_ERR_ALIGN: return "q/k/v rows must be 16-byte aligned and o rows 8-byte aligned";

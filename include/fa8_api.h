@@ -27,7 +27,8 @@ extern "C" {
 
 /* element types of o */
 #define FA8_OUT_FP16 0 /* IEEE half, round-to-nearest-even */
-#define FA8_OUT_E4M3 1 /* e4m3fn, RNE, saturate-to-finite: what the reference stores (csrc/flash_attention.cu:557,656) */
+#define FA8_OUT_E4M3 1 /* e4m3fn, RNE, saturate-to-finite: what the reference stores (csrc/flash_attention.cu:557,656); e4m3 inputs only */
+#define FA8_OUT_E5M2 2 /* e5m2, RNE, saturate-to-finite: the reference's output for e5m2 inputs (same lines); e5m2 inputs only */
 
 /* layouts of v */
 #define FA8_V_ROWS 0       /* v is [B,H,Nk,d]: same as k */
@@ -59,7 +60,7 @@ typedef struct Fa8FwdParams {
   const void* q; /* [B,H,Nq,d] fp8 */
   const void* k; /* [B,Hk,Nk,d] fp8; Hk = heads_k (or heads) */
   const void* v; /* [B,Hk,Nk,d] fp8 (FA8_V_ROWS) or [B,Hk,d,Nk] (FA8_V_TRANSPOSED) */
-  void* o;       /* [B,H,Nq,d] fp16 or e4m3 */
+  void* o;       /* [B,H,Nq,d] fp16, or fp8 of the input element type */
   int32_t batch;
   int32_t heads;
   int32_t seqlen_q;
