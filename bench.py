@@ -118,6 +118,10 @@ def main():
                     help="instead of the headline step, time the 18 shapes of the reference's own benchmark table "
                          "(reference test.py:95-100: B=1, causal, scale=1/sqrt(N), inputs clamped to +-0.1) and print "
                          "one JSON line holding the table next to the reference's published Ada numbers")
+    ap.add_argument("--instruction-mix", action="store_true",
+                    help="run only the instruction-mix probe (cutlass_flash_atten_fp8_amd/csrc/softmax_mix_probe.hip): what a "
+                         "SIMD needs for the vector and matrix instructions of one KV block with no memory traffic at all; "
+                         "prints its JSON lines")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a plain 256 MiB device-to-device copy (10 times): the known-size kernel that the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run are scaled by")
@@ -127,6 +131,12 @@ def main():
               "see DESIGN.md); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
 
+    if args.instruction_mix:
+        import subprocess
+        from cutlass_flash_atten_fp8_amd import build as native_build
+        if not os.path.exists(native_build.MIX_PROBE):
+            native_build.build_mix_probe()
+        sys.exit(subprocess.run([native_build.MIX_PROBE]).returncode)
     import torch
     import cutlass_flash_atten_fp8_amd as fa
     from cutlass_flash_atten_fp8_amd import inputs
