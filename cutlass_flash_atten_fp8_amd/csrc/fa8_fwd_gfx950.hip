@@ -58,6 +58,7 @@ struct KernelArgs {
   float* lse;  // optional
   int heads, seqlen_q, seqlen_k, n_qblocks, bh_total;
   int kv_group;      // q heads per k/v head
+  int interleave;    // causal: how many heads deal their q blocks alternately (see decode_block)
   int causal_shift;  // key j is visible to query i when j <= i + causal_shift
   float scale_log2;  // softmax_scale * log2(e)
   long long q_bs, q_hs, q_rs;
@@ -164,19 +165,37 @@ __device__ __forceinline__ int pack4_fp8(float a, float b, float c, float d) {
 
 // Workgroup id -> (batch*head, q block).  Workgroups are dealt to the 8 XCDs round-robin by id; when
 // batch*heads is a multiple of 8 all q blocks of one head are kept on one XCD so its K/V stay in that
-// XCD's L2.  Causal problems start with the longest (last) q blocks.
+// XCD's L2.  Workgroups start in id order.  Full attention: head after head.  Causal: workgroups differ in length
+// (q block i walks i+1 of the n q blocks' worth of keys), so the longest come first and `interleave` heads of the XCD
+// take turns at every q block: the workgroups that run side by side then have about the same length and the
+// short ones fill the end of the launch (head after head, a late head's longest workgroup would start when the
+// rest of the chip is already draining).
 template <bool CAUSAL>
 __device__ __forceinline__ void decode_block(const KernelArgs& a, int id, int& bh, int& qb) {
   int qi;
   if ((a.bh_total & 7) == 0) {
     const int xcd = id & 7, s = id >> 3;
+    int hl;  // head index inside this XCD's share of bh_total / 8 heads
+    if (CAUSAL) {
+      // groups of `interleave` heads (the last group takes what is left)
+      const int per_group = a.interleave * a.n_qblocks;
+      const int grp = s / per_group, r = s - grp * per_group;
+      const int g = min(a.interleave, (a.bh_total >> 3) - grp * a.interleave);
+      qi = r / g;
+      hl = grp * a.interleave + (r - qi * g);
+    } else {
+      hl = s / a.n_qblocks;
+      qi = s - hl * a.n_qblocks;
+    }
     // grouped-query attention: an XCD takes a contiguous range of q heads, so the heads that share a k/v head follow
     // each other on one XCD
-    bh = a.kv_group > 1 ? xcd * (a.bh_total >> 3) + s / a.n_qblocks : (s / a.n_qblocks) * 8 + xcd;
-    qi = s % a.n_qblocks;
+    bh = a.kv_group > 1 ? xcd * (a.bh_total >> 3) + hl : hl * 8 + xcd;
+  } else if (CAUSAL) {
+    qi = id / a.bh_total;  // no head stays on one XCD anyway: all heads take turns
+    bh = id - qi * a.bh_total;
   } else {
     bh = id / a.n_qblocks;
-    qi = id % a.n_qblocks;
+    qi = id - bh * a.n_qblocks;
   }
   qb = CAUSAL ? (a.n_qblocks - 1 - qi) : qi;
 }
@@ -661,6 +680,7 @@ extern "C" int fa8_fwd(const Fa8FwdParams* p, void* hip_stream) {
   a.seqlen_k = p->seqlen_k;
   a.n_qblocks = (p->seqlen_q + kQBlock - 1) / kQBlock;
   a.bh_total = p->batch * p->heads;
+  a.interleave = a.bh_total / 8 < 8 ? (a.bh_total / 8 > 0 ? a.bh_total / 8 : 1) : 8;  // causal launches, see decode_block
   a.scale_log2 = p->softmax_scale * 1.4426950408889634f;
   a.q_bs = p->q_batch_stride; a.q_hs = p->q_head_stride; a.q_rs = p->q_row_stride;
   a.k_bs = p->k_batch_stride; a.k_hs = p->k_head_stride; a.k_rs = p->k_row_stride;
