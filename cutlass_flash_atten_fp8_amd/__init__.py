@@ -26,6 +26,7 @@ FA8_DTYPE_E4M3, FA8_DTYPE_E5M2 = 0, 1
 FA8_OUT_FP16, FA8_OUT_E4M3, FA8_OUT_E5M2 = 0, 1, 2
 FA8_V_ROWS, FA8_V_TRANSPOSED = 0, 1
 FA8_CAUSAL_TOP_LEFT, FA8_CAUSAL_BOTTOM_RIGHT = 0, 1
+FA8_SCHEDULE_AUTO, FA8_SCHEDULE_ROLLING, FA8_SCHEDULE_PIPELINED = 0, 1, 2
 (FA8_QUERY_VERSION, FA8_QUERY_KV_BLOCK, FA8_QUERY_Q_BLOCK, FA8_QUERY_KV_ASCENDING, FA8_QUERY_THREADS,
  FA8_QUERY_PARAMS_SIZE) = range(6)
 FA8_EXPORTS = ("fa8_fwd_validate", "fa8_fwd", "fa8_query", "fa8_error_string")
@@ -45,6 +46,7 @@ class Fa8FwdParams(ctypes.Structure):
         ("o_batch_stride", ctypes.c_int64), ("o_head_stride", ctypes.c_int64), ("o_row_stride", ctypes.c_int64),
         ("lse", ctypes.c_void_p), ("lse_batch_stride", ctypes.c_int64), ("lse_head_stride", ctypes.c_int64),
         ("heads_k", ctypes.c_int32), ("causal_align", ctypes.c_int32),
+        ("schedule", ctypes.c_int32), ("reserved0", ctypes.c_int32),
     ]
 
 
@@ -94,7 +96,8 @@ def load_extension():
     return mod
 
 
-def make_params(q, k, v, o, is_causal, softmax_scale, v_transposed=False, lse=None, causal_bottom_right=False):
+def make_params(q, k, v, o, is_causal, softmax_scale, v_transposed=False, lse=None, causal_bottom_right=False,
+                schedule=0):
     """Fill Fa8FwdParams from torch tensors (any device: only shapes, strides and pointers are read).
     k and v may have fewer heads than q (grouped-query attention); lse, if given, is a float32 [B,H,Nq] output."""
     import torch
@@ -126,6 +129,7 @@ def make_params(q, k, v, o, is_causal, softmax_scale, v_transposed=False, lse=No
         setattr(p, name + "_row_stride", t.stride(2))
     p.heads_k = k.shape[1]
     p.causal_align = FA8_CAUSAL_BOTTOM_RIGHT if causal_bottom_right else FA8_CAUSAL_TOP_LEFT
+    p.schedule = int(schedule)
     if lse is not None:
         if lse.dtype != torch.float32 or lse.dim() != 3 or lse.stride(2) != 1:
             raise RuntimeError("lse must be a float32 [batch, heads, seqlen_q] tensor with contiguous rows")
@@ -134,7 +138,7 @@ def make_params(q, k, v, o, is_causal, softmax_scale, v_transposed=False, lse=No
 
 
 def flash_attention_v2_cutlass(q, k, v, is_causal, softmax_scale, *, v_transposed=False, out_dtype=None, return_lse=False,
-                               causal_bottom_right=False):
+                               causal_bottom_right=False, schedule=0):
     """The reference operator (reference csrc/flash_attention.cu:639-668) through the C ABI.
 
     q, k: fp8 [B,H,N,d] on the GPU; v: [B,H,N,d] (or [B,H,d,N] with v_transposed=True, as the reference
@@ -143,7 +147,8 @@ def flash_attention_v2_cutlass(q, k, v, is_causal, softmax_scale, *, v_transpose
     RuntimeError on bad arguments, like the reference's TORCH_CHECKs (include/attention_api.cuh:12-18).
     Beyond the reference: k/v may have fewer heads than q (grouped-query attention), return_lse=True returns
     [O, lse] with lse the float32 [B,H,Nq] log-sum-exp of the scaled logits, causal_bottom_right=True aligns the
-    causal diagonal with the last key when seqlen_q != seqlen_k.
+    causal diagonal with the last key when seqlen_q != seqlen_k; schedule (FA8_SCHEDULE_*) is a performance hint that
+    never changes the result.
     """
     import torch
     for name, t in (("q", q), ("k", k), ("v", v)):
@@ -166,7 +171,7 @@ def flash_attention_v2_cutlass(q, k, v, is_causal, softmax_scale, *, v_transpose
         raise RuntimeError("q, k and v must be on the same device")
     o = torch.empty((B, H, Nq, D), dtype=out_dtype or torch.float16, device=q.device)
     lse = torch.empty((B, H, Nq), dtype=torch.float32, device=q.device) if return_lse else None
-    p = make_params(q, k, v, o, is_causal, softmax_scale, v_transposed, lse, causal_bottom_right)
+    p = make_params(q, k, v, o, is_causal, softmax_scale, v_transposed, lse, causal_bottom_right, schedule)
     with torch.cuda.device(q.device):
         stream = torch.cuda.current_stream(q.device).cuda_stream
         rc = lib().fa8_fwd(ctypes.byref(p), ctypes.c_void_p(stream))

@@ -66,7 +66,8 @@ CABI_HOST = os.path.join(os.path.dirname(PKG_DIR), "tests", "cabi_host")
 
 def build_cabi_host(force=False):
     """tests/cabi_host: the standalone C++ host of the C ABI used by tests/test_cabi_host_gpu.py (host code only)."""
-    if force or not os.path.exists(CABI_HOST) or os.path.getmtime(CABI_HOST) < os.path.getmtime(CABI_HOST_SRC):
+    newest = max(os.path.getmtime(CABI_HOST_SRC), os.path.getmtime(os.path.join(INCLUDE, "fa8_api.h")))
+    if force or not os.path.exists(CABI_HOST) or os.path.getmtime(CABI_HOST) < newest:
         _run(["g++", "-O2", "-std=c++17", "-D__HIP_PLATFORM_AMD__=1", "-I", INCLUDE, "-I", os.path.join(ROCM, "include"),
               CABI_HOST_SRC, "-o", CABI_HOST, "-L", PKG_DIR, "-l:libfa8.so", "-L", os.path.join(ROCM, "lib"), "-lamdhip64",
               "-Wl,-rpath," + PKG_DIR, "-Wl,-rpath," + os.path.join(ROCM, "lib")])

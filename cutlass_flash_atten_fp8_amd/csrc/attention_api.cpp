@@ -12,7 +12,8 @@
 //   * bad arguments and HIP errors raise RuntimeError instead of printf + exit (include/attention_api.cuh:20-29).
 // Additions the reference declares but never implements (csrc/flash.h:36-45,56): k/v may have fewer heads than q
 // (grouped-query attention), `return_lse=True` appends the fp32 log-sum-exp [B,H,Nq] to the returned list, and
-// `causal_bottom_right=True` aligns the causal diagonal with the last key when seqlen_q != seqlen_k.
+// `causal_bottom_right=True` aligns the causal diagonal with the last key when seqlen_q != seqlen_k.  `schedule`
+// (FA8_SCHEDULE_*, include/fa8_api.h) picks the kernel's main loop by hand: a performance hint, the result is the same.
 #include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <torch/extension.h>
@@ -35,7 +36,7 @@ void check_input(const torch::Tensor& t, const char* name) {
 std::vector<torch::Tensor> flash_attention_v2_cutlass(torch::Tensor q, torch::Tensor k, torch::Tensor v, bool is_causal,
                                                       float softmax_scale, bool v_transposed,
                                                       c10::optional<at::ScalarType> out_dtype, bool return_lse,
-                                                      bool causal_bottom_right) {
+                                                      bool causal_bottom_right, int64_t schedule) {
   check_input(q, "q");
   check_input(k, "k");
   check_input(v, "v");
@@ -86,6 +87,7 @@ std::vector<torch::Tensor> flash_attention_v2_cutlass(torch::Tensor q, torch::Te
   p.o_batch_stride = out.stride(0); p.o_head_stride = out.stride(1); p.o_row_stride = out.stride(2);
   p.heads_k = (int32_t)Hk;
   p.causal_align = causal_bottom_right ? FA8_CAUSAL_BOTTOM_RIGHT : FA8_CAUSAL_TOP_LEFT;
+  p.schedule = (int32_t)schedule;
   if (return_lse) {
     p.lse = lse.data_ptr();
     p.lse_batch_stride = lse.stride(0);
@@ -106,6 +108,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("flash_attention_v2_cutlass", &flash_attention_v2_cutlass,
         "FP8 flash attention forward: fp8 q/k/v [B,H,N,d] -> [O] (fp16 by default)", py::arg("q"), py::arg("k"),
         py::arg("v"), py::arg("is_causal"), py::arg("softmax_scale"), py::kw_only(), py::arg("v_transposed") = false,
-        py::arg("out_dtype") = py::none(), py::arg("return_lse") = false, py::arg("causal_bottom_right") = false);
+        py::arg("out_dtype") = py::none(), py::arg("return_lse") = false, py::arg("causal_bottom_right") = false,
+        py::arg("schedule") = 0);
   m.def("kv_block", []() { return fa8_query(FA8_QUERY_KV_BLOCK); }, "kv rows per online-softmax step of the kernel");
 }

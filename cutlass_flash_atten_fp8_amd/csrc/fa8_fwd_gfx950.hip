@@ -48,7 +48,7 @@ constexpr int kQBlock = 128;   // query rows per workgroup
 constexpr int kQWave = 32;     // query rows per wavefront
 constexpr int kKvBlock = 64;   // kv rows per online-softmax step
 constexpr int kThreads = 256;  // 4 wavefronts
-constexpr int kVersion = 2;
+constexpr int kVersion = 3;
 
 struct KernelArgs {
   const uint8_t* q;
@@ -200,8 +200,14 @@ __device__ __forceinline__ void decode_block(const KernelArgs& a, int id, int& b
   qb = CAUSAL ? (a.n_qblocks - 1 - qi) : qi;
 }
 
-template <int D, bool CAUSAL, bool E5M2, int OUT, bool VT>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WAVES_PER_EU(D)))) void fa8_fwd_kernel(
+// PIPE selects the main loop.  false: one KV block after the other (S^T, softmax, PV), three wavefronts per SIMD hide each
+// other's latencies: the loop for launches that fill the chip.  true: a software-pipelined loop for launches that leave
+// a SIMD with two wavefronts or fewer (short sequences, few heads): the matrix instructions of the neighbouring blocks
+// (PV of block j-1, S^T of block j+1) are issued between the chunks of the softmax of block j, so that one wavefront alone
+// keeps the matrix and the vector pipe busy; it needs about 200 VGPRs (two wavefronts per SIMD) and four LDS stages.
+// Both loops perform the same arithmetic in the same order: their results are bitwise equal.
+template <int D, bool CAUSAL, bool E5M2, int OUT, bool VT, bool PIPE>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PIPE ? 2 : FA8_WAVES_PER_EU(D)))) void fa8_fwd_kernel(
     const KernelArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the body uses device-only types (buffer resources); the host pass only needs the stub
   static_assert(D % 32 == 0 && D >= 32 && D <= 256, "head dims: multiples of 32 up to 256");
@@ -216,15 +222,18 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
   constexpr int kMTiles = D / 32;         // 32-row tiles of O^T
   // LDS stages per operand: three (copies issued two KV blocks ahead) where three workgroups then still fit in the
   // 160 KB of a CU, two for head dims above 128 (2 x 32 KB per workgroup, two workgroups per CU)
-  constexpr int kStages = D > 128 ? 2 : 3;
+  // (the pipelined loop: four, copies issued up to four blocks ahead)
+  constexpr int kStages = PIPE ? 4 : (D > 128 ? 2 : 3);
   // One LDS object per (stage, operand): the compiler then knows that the asynchronous HBM -> LDS copy into one
   // stage cannot alias the reads of the other stage and does not wait for the copy before those reads.
   __shared__ __attribute__((aligned(1024))) uint8_t k_lds0[kTileBytes];
   __shared__ __attribute__((aligned(1024))) uint8_t k_lds1[kTileBytes];
-  __shared__ __attribute__((aligned(1024))) uint8_t k_lds2[kStages == 3 ? kTileBytes : 16];
+  __shared__ __attribute__((aligned(1024))) uint8_t k_lds2[kStages >= 3 ? kTileBytes : 16];
+  __shared__ __attribute__((aligned(1024))) uint8_t k_lds3[kStages >= 4 ? kTileBytes : 16];
   __shared__ __attribute__((aligned(1024))) uint8_t v_lds0[kTileBytes];
   __shared__ __attribute__((aligned(1024))) uint8_t v_lds1[kTileBytes];
-  __shared__ __attribute__((aligned(1024))) uint8_t v_lds2[kStages == 3 ? kTileBytes : 16];
+  __shared__ __attribute__((aligned(1024))) uint8_t v_lds2[kStages >= 3 ? kTileBytes : 16];
+  __shared__ __attribute__((aligned(1024))) uint8_t v_lds3[kStages >= 4 ? kTileBytes : 16];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keep it (and all it feeds) in scalar registers
@@ -290,9 +299,15 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
       __builtin_amdgcn_make_buffer_rsrc((void*)kp, 0, (int)(kv_last * a.k_rs + D), kRsrcFlags);
   const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(
       (void*)vp, 0, VT ? (int)((D - 1) * a.v_rs + a.seqlen_k) : (int)(kv_last * a.v_rs + D), kRsrcFlags);
-  // Start the asynchronous copy of KV block j into the LDS buffers kb / vb.
-  auto issue_tile = [&](int j, uint8_t* kb, uint8_t* vb) __attribute__((always_inline)) {
+  // Start the asynchronous copy of the K rows / the V rows of KV block j into the LDS buffer kb / vb.
+  auto issue_k = [&](int j, uint8_t* kb) __attribute__((always_inline)) {
     const int k_base = j * kKvBlock * (int)a.k_rs;
+#pragma unroll
+    for (int p = 0; p < kPasses; ++p)
+      if (!kSplitPass || wave < 2)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, LDS_PTR(void, kb + copy_segment(p) * 1024), 16, k_src[p], k_base, 0, 0);
+  };
+  auto issue_v = [&](int j, uint8_t* vb) __attribute__((always_inline)) {
     const int v_base = VT ? j * kKvBlock : j * kKvBlock * (int)a.v_rs;
     // transposed v, ragged last block: the 16-byte chunks past the last kv column would read the start of the next
     // head-dim row (or run off the tensor); they are pulled back onto the last chunk instead (and masked later)
@@ -300,8 +315,6 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
 #pragma unroll
     for (int p = 0; p < kPasses; ++p) {
       const int seg = copy_segment(p) * 1024;
-      if (!kSplitPass || wave < 2)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, LDS_PTR(void, kb + seg), 16, k_src[p], k_base, 0, 0);
       if (!kSplitPass || wave >= 2) {
         if (v_clamp) {
           int r, ch;
@@ -313,6 +326,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
         }
       }
     }
+  };
+  auto issue_tile = [&](int j, uint8_t* kb, uint8_t* vb) __attribute__((always_inline)) {
+    issue_k(j, kb);
+    issue_v(j, vb);
   };
 
   // ---- per-lane LDS read offsets ----
@@ -357,6 +374,29 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
   float m_run = -INFINITY;  // running row max of raw S (both half-lanes of a query hold the same value)
   float l_run = 0.f;        // this lane's share of the running row sum
 
+  // K fragment of S^T sub-tile t, k-step ks, and V^T fragment of O^T tile mt, from the tiles in kb / vb
+  auto load_kf = [&](const uint8_t* kb, int t, int ks) __attribute__((always_inline)) {
+    const v4i lo = *LDS_PTR(const v4i, kb + t * kSubTileStride + k_off[ks][0]);
+    const v4i hi = *LDS_PTR(const v4i, kb + t * kSubTileStride + k_off[ks][1]);
+    return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  };
+  auto load_vf = [&](const uint8_t* vb, int mt) __attribute__((always_inline)) {
+    v8i vf;
+    if constexpr (VT) {
+      const v4i lo = *LDS_PTR(const v4i, vb + mt * kVtTileStride + vt_off[0]);
+      const v4i hi = *LDS_PTR(const v4i, vb + mt * kVtTileStride + vt_off[1]);
+      vf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    } else {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const v2i r = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_PTR(v2i, vb + v_off[mt] + g * kTrStride));
+        vf[2 * g] = r[0];
+        vf[2 * g + 1] = r[1];
+      }
+    }
+    return vf;
+  };
+
   // S^T, online softmax and PV for KV block j held in kb / vb.
   auto compute_tile = [&](int j, const uint8_t* kb, const uint8_t* vb, auto masked_c) __attribute__((always_inline)) {
     // kMasked also marks the general path (first block, diagonal, tail): only there can the running max still be -inf
@@ -370,10 +410,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
       for (int i = 0; i < 16; ++i) s[t][i] = 0.f;
 #pragma unroll
       for (int ks = 0; ks < kKSteps; ++ks) {
-        const v4i lo = *LDS_PTR(const v4i, kb + t * kSubTileStride + k_off[ks][0]);
-        const v4i hi = *LDS_PTR(const v4i, kb + t * kSubTileStride + k_off[ks][1]);
-        const v8i kf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        s[t] = mfma_fp8<E5M2>(kf, qf[ks], s[t]);
+        s[t] = mfma_fp8<E5M2>(load_kf(kb, t, ks), qf[ks], s[t]);
       }
     }
     // ---- causal / tail mask: register i of sub-tile t is kv row kv0 + 32h + 16t + i ----
@@ -431,27 +468,11 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
     }
     l_run += sum0 + sum1;
     // ---- O^T += V^T P^T : the V^T fragment of tile mt+1 is fetched while the MFMA of tile mt runs ----
-    auto load_vf = [&](int mt) __attribute__((always_inline)) {
-      v8i vf;
-      if constexpr (VT) {
-        const v4i lo = *LDS_PTR(const v4i, vb + mt * kVtTileStride + vt_off[0]);
-        const v4i hi = *LDS_PTR(const v4i, vb + mt * kVtTileStride + vt_off[1]);
-        vf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-      } else {
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const v2i r = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_PTR(v2i, vb + v_off[mt] + g * kTrStride));
-          vf[2 * g] = r[0];
-          vf[2 * g + 1] = r[1];
-        }
-      }
-      return vf;
-    };
-    v8i vf_cur = load_vf(0);
+    v8i vf_cur = load_vf(vb, 0);
 #pragma unroll
     for (int mt = 0; mt < kMTiles; ++mt) {
       v8i vf_next;
-      if (mt + 1 < kMTiles) vf_next = load_vf(mt + 1);
+      if (mt + 1 < kMTiles) vf_next = load_vf(vb, mt + 1);
       o_acc[mt] = mfma_fp8<E5M2>(vf_cur, p8, o_acc[mt]);
       if (mt + 1 < kMTiles) vf_cur = vf_next;
     }
@@ -472,7 +493,193 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
   };
   static_assert(kLoadsPerTile < 16, "vmcnt immediate above");
 
-  if constexpr (kStages == 3) {
+  if constexpr (PIPE) {
+    // ---- software-pipelined loop ----
+    // Iteration j is the softmax of block j in 8 chunks of 4 weights with a matrix instruction in front of the chunks: first
+    // the PV products of block j-1, then the S^T products of block j+1 (head dim 128: one per chunk, 64: every second
+    // chunk), their LDS operands fetched two instructions ahead.  K(t) lives in K stage t % 4, V(t) in V stage t % 4.  Step j
+    // starts the copies of K(j+4) and V(j+2) (their stages held K(j) and V(j-2), last read in iteration j-1), reads K(j+1)
+    // and V(j-1), and ends when K(j+2) and V(j) have landed.  Every block takes this path, masked blocks included (their
+    // weights become exact zeros), so the loop needs no second form.
+    static_assert(!PIPE || D == 64 || D == 128, "the pipelined loop is built for head dims 64 and 128");
+    constexpr int kSlots = kMTiles + 2 * kKSteps;  // matrix instructions per iteration
+    constexpr int kChunksPerSlot = 8 / kSlots;     // 1 (head dim 128) or 2 (64)
+    v16f sbuf[2][2];
+    v8i p8buf[2];
+    const int kv_limit = CAUSAL ? min(q_row + shift, kv_last) : kv_last;  // last kv this query attends to
+    auto iteration = [&](auto first_c, int j, const uint8_t* kb_next, const uint8_t* vb_prev, v16f(&s)[2], v16f(&sn)[2],
+                         const v8i& p8_prev, v8i& p8_cur) __attribute__((always_inline)) {
+      constexpr bool kFirst = decltype(first_c)::value;
+      const bool masked = j >= n_plain;  // wave-uniform
+      v8i frag[kSlots];
+      if constexpr (!kFirst) {
+        frag[0] = load_vf(vb_prev, 0);
+        frag[1] = load_vf(vb_prev, 1);
+      }
+      if (masked) {
+        // a masked logit becomes -inf and its weight exp2(-inf) = 0 (the launcher takes this loop only for scale > 0)
+        const int kv0 = j * kKvBlock;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int i = 0; i < 16; ++i)
+            if (kv0 + 32 * h + 16 * t + i > kv_limit) s[t][i] = -INFINITY;
+      }
+      float mx[4];
+#pragma unroll
+      for (int ch = 0; ch < 4; ++ch) mx[ch] = max3(s[0][4 * ch], s[0][4 * ch + 1], s[0][4 * ch + 2]);
+#pragma unroll
+      for (int ch = 0; ch < 4; ++ch) mx[ch] = max3(mx[ch], s[0][4 * ch + 3], s[1][4 * ch]);
+#pragma unroll
+      for (int ch = 0; ch < 4; ++ch) mx[ch] = max3(mx[ch], s[1][4 * ch + 1], s[1][4 * ch + 2]);
+      const float m_new = lane32_max(max3(max3(mx[0], s[1][3], s[1][7]), max3(mx[1], s[1][11], s[1][15]), max3(mx[2], mx[3], m_run)));
+      bool changed = false;
+      float alpha = 1.f;
+      float mc = m_new * c;
+      if constexpr (kFirst) {
+        m_run = m_new;  // O and l are still zero
+      } else {
+        changed = __any(m_new != m_run);
+        if (changed) {
+          alpha = __builtin_amdgcn_exp2f((m_run - m_new) * c);
+          if (masked) alpha = (m_run == -INFINITY) ? 0.f : alpha;  // a row that has not seen a key yet
+          l_run *= alpha;
+          m_run = m_new;
+        }
+      }
+      if (masked) mc = (m_new == -INFINITY) ? 0.f : mc;
+      float sum0, sum1;
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        if (u % kChunksPerSlot == 0) {
+          const int slot = u / kChunksPerSlot;
+          // operands of the matrix instruction two slots ahead
+          if (slot + 2 < kSlots) {
+            const int sl = slot + 2;
+            if (sl < kMTiles) {
+              if constexpr (!kFirst) frag[sl] = load_vf(vb_prev, sl);
+            } else {
+              frag[sl] = load_kf(kb_next, (sl - kMTiles) / kKSteps, (sl - kMTiles) % kKSteps);
+            }
+          }
+          if (slot < kMTiles) {
+            if constexpr (!kFirst) o_acc[slot] = mfma_fp8<E5M2>(frag[slot], p8_prev, o_acc[slot]);
+          } else {
+            // (after the last block this is the product of a stale tile: never used)
+            const int t = (slot - kMTiles) / kKSteps, ks = (slot - kMTiles) % kKSteps;
+            if (ks == 0) {
+              v16f z;
+#pragma unroll
+              for (int i = 0; i < 16; ++i) z[i] = 0.f;
+              sn[t] = mfma_fp8<E5M2>(frag[slot], qf[ks], z);
+            } else {
+              sn[t] = mfma_fp8<E5M2>(frag[slot], qf[ks], sn[t]);
+            }
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        // chunk u of the softmax: weights 4w .. 4w+3 of sub-tile t
+        const int t = u >> 2, w = u & 3;
+#pragma unroll
+        for (int i = 4 * w; i < 4 * w + 4; ++i) s[t][i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][i], c, -mc));
+        sum0 = (u == 0) ? s[t][4 * w] : sum0 + s[t][4 * w];
+        sum1 = (u == 0) ? s[t][4 * w + 1] : sum1 + s[t][4 * w + 1];
+        sum0 += s[t][4 * w + 2];
+        sum1 += s[t][4 * w + 3];
+        p8_cur[u] = pack4_fp8<E5M2>(s[t][4 * w], s[t][4 * w + 1], s[t][4 * w + 2], s[t][4 * w + 3]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      l_run += sum0 + sum1;
+      asm volatile("" : "+v"(l_run));  // keeps the additions above where they are written (sunk to the end they cost registers)
+      // O now holds the PV product of block j-1 (issued four or more chunks ago): bring it to the new row max
+      if (changed) {
+#pragma unroll
+        for (int mt = 0; mt < kMTiles; ++mt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) o_acc[mt][i] *= alpha;
+      }
+    };
+    // Every step starts two tile copies, also past the last block (those read beyond the buffer: zeros, no memory traffic,
+    // never used), so the number of loads in flight is the same at every step.  vmcnt counts this lane's loads in issue order.
+    // Waits until at most `tiles` tile copies (kPasses loads each) are in flight, then the barrier: it publishes the landed
+    // tiles and frees the stages read before it.
+    auto wait_in_flight = [&](auto tiles_c) __attribute__((always_inline)) {
+      constexpr int n = decltype(tiles_c)::value * kPasses;
+      static_assert(n < 16, "vmcnt immediate");
+      __builtin_amdgcn_s_waitcnt(0x0F70 | n);
+      __builtin_amdgcn_s_barrier();
+    };
+    // Ends step j: K(j+2) and V(j) must have landed; the copies of steps j-1 and j (K(j+3), V(j+1), K(j+4), V(j+2)) may stay
+    // in flight.
+    auto end_step = [&]() __attribute__((always_inline)) { wait_in_flight(std::integral_constant<int, 4>()); };
+    // The PV product of the last block (its weights are in p8), V in stage vb.
+    auto finish = [&](const uint8_t* vb, const v8i& p8) __attribute__((always_inline)) {
+#pragma unroll
+      for (int mt = 0; mt < kMTiles; ++mt) o_acc[mt] = mfma_fp8<E5M2>(load_vf(vb, mt), p8, o_acc[mt]);
+    };
+    using T = std::true_type;
+    using F = std::false_type;
+    // the copies of steps -4 .. -1
+    issue_k(0, k_lds0);
+    issue_k(1, k_lds1);
+    issue_k(2, k_lds2);
+    issue_v(0, v_lds0);
+    issue_k(3, k_lds3);
+    issue_v(1, v_lds1);
+    wait_in_flight(std::integral_constant<int, 5>());  // K(0) landed
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) sbuf[0][t][i] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < kKSteps; ++ks) sbuf[0][t] = mfma_fp8<E5M2>(load_kf(k_lds0, t, ks), qf[ks], sbuf[0][t]);
+    }
+    end_step();  // K(1) landed, and every wavefront has read K(0): step 0 may overwrite its stage
+    // One step with compile-time LDS stages (PH = j % 4) and buffers (j % 2); the mask-free form for the leading blocks.
+    auto step = [&](auto first_c, auto ph_c, int j) __attribute__((always_inline)) {
+      constexpr int PH = decltype(ph_c)::value;
+      constexpr bool kFirst = decltype(first_c)::value;
+      uint8_t* const kst[4] = {k_lds0, k_lds1, k_lds2, k_lds3};
+      uint8_t* const vst[4] = {v_lds0, v_lds1, v_lds2, v_lds3};
+      issue_k(j + 4, kst[PH]);
+      issue_v(j + 2, vst[(PH + 2) % 4]);
+      iteration(first_c, j, kst[(PH + 1) % 4], vst[(PH + 3) % 4], sbuf[PH % 2], sbuf[(PH + 1) % 2], p8buf[(PH + 1) % 2],
+                p8buf[PH % 2]);
+      end_step();
+      (void)kFirst;
+    };
+    constexpr std::integral_constant<int, 0> ph0{};
+    constexpr std::integral_constant<int, 1> ph1{};
+    constexpr std::integral_constant<int, 2> ph2{};
+    constexpr std::integral_constant<int, 3> ph3{};
+    step(T(), ph0, 0);
+    int j = 1;
+    for (; j + 3 < n_tiles; j += 4) {
+      step(F(), ph1, j);
+      step(F(), ph2, j + 1);
+      step(F(), ph3, j + 2);
+      step(F(), ph0, j + 3);
+    }
+    // up to three more blocks; the weights of the last block end in p8buf[0]
+    if (j < n_tiles) {
+      step(F(), ph1, j);
+      if (j + 1 < n_tiles) {
+        step(F(), ph2, j + 1);
+        if (j + 2 < n_tiles) {
+          step(F(), ph3, j + 2);
+          p8buf[0] = p8buf[1];
+        }
+      } else {
+        p8buf[0] = p8buf[1];
+      }
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // the copies past the last block must not outlive the workgroup's LDS
+    {
+      const int st = (n_tiles - 1) & 3;
+      finish(st == 0 ? v_lds0 : (st == 1 ? v_lds1 : (st == 2 ? v_lds2 : v_lds3)), p8buf[0]);
+    }
+  } else if constexpr (kStages == 3) {
     issue_tile(0, k_lds0, v_lds0);
     if (n_tiles > 1) issue_tile(1, k_lds1, v_lds1);
     stage_sync(n_tiles > 1);
@@ -590,26 +797,46 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
 }
 
 template <int D, bool CAUSAL, bool E5M2, int OUT>
-int launch(const KernelArgs& a, bool v_transposed, hipStream_t stream) {
+int launch(const KernelArgs& a, bool v_transposed, bool pipelined, hipStream_t stream) {
   const dim3 grid((unsigned)(a.bh_total * a.n_qblocks));
   // hipLaunchKernel returns the status of this launch itself; the thread's sticky "last error" (which an earlier,
   // unrelated call may have left behind) is neither read nor cleared.
   KernelArgs args = a;
   void* argv[] = {&args};
-  const void* fn = v_transposed ? (const void*)&fa8_fwd_kernel<D, CAUSAL, E5M2, OUT, true>
-                                : (const void*)&fa8_fwd_kernel<D, CAUSAL, E5M2, OUT, false>;
+  const void* fn = v_transposed ? (const void*)&fa8_fwd_kernel<D, CAUSAL, E5M2, OUT, true, false>
+                                : (const void*)&fa8_fwd_kernel<D, CAUSAL, E5M2, OUT, false, false>;
+  if constexpr (D == 64 || D == 128) {
+    if (pipelined)
+      fn = v_transposed ? (const void*)&fa8_fwd_kernel<D, CAUSAL, E5M2, OUT, true, true>
+                        : (const void*)&fa8_fwd_kernel<D, CAUSAL, E5M2, OUT, false, true>;
+  }
   return (int)hipLaunchKernel(fn, grid, dim3(kThreads), argv, 0, stream);
 }
 
 template <int D, bool CAUSAL>
-int launch_types(const Fa8FwdParams* p, const KernelArgs& a, hipStream_t stream) {
+int launch_types(const Fa8FwdParams* p, const KernelArgs& a, bool pipelined, hipStream_t stream) {
   const bool e5m2 = p->in_dtype == FA8_DTYPE_E5M2, vt = p->v_layout == FA8_V_TRANSPOSED;
   if (p->out_dtype == FA8_OUT_FP16)
-    return e5m2 ? launch<D, CAUSAL, true, FA8_OUT_FP16>(a, vt, stream) : launch<D, CAUSAL, false, FA8_OUT_FP16>(a, vt, stream);
+    return e5m2 ? launch<D, CAUSAL, true, FA8_OUT_FP16>(a, vt, pipelined, stream)
+                : launch<D, CAUSAL, false, FA8_OUT_FP16>(a, vt, pipelined, stream);
   // fp8 output: the reference stores O in the input element type (csrc/flash_attention.cu:557, :655-656); the two
   // mixed combinations are not built
-  if (e5m2) return p->out_dtype == FA8_OUT_E5M2 ? launch<D, CAUSAL, true, FA8_OUT_E5M2>(a, vt, stream) : FA8_ERR_UNSUPPORTED;
-  return p->out_dtype == FA8_OUT_E4M3 ? launch<D, CAUSAL, false, FA8_OUT_E4M3>(a, vt, stream) : FA8_ERR_UNSUPPORTED;
+  if (e5m2)
+    return p->out_dtype == FA8_OUT_E5M2 ? launch<D, CAUSAL, true, FA8_OUT_E5M2>(a, vt, pipelined, stream) : FA8_ERR_UNSUPPORTED;
+  return p->out_dtype == FA8_OUT_E4M3 ? launch<D, CAUSAL, false, FA8_OUT_E4M3>(a, vt, pipelined, stream) : FA8_ERR_UNSUPPORTED;
+}
+
+// Compute units of the current device (0 if the runtime cannot tell), asked once per device.
+int compute_units() {
+  static int cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1) return 0;
+    cached[dev] = n;
+  }
+  return cached[dev];
 }
 
 bool span_ok(long long outer_stride, long long inner_extent) { return outer_stride >= inner_extent; }
@@ -622,6 +849,8 @@ extern "C" int fa8_fwd_validate(const Fa8FwdParams* p) {
   if (p->is_causal != 0 && p->is_causal != 1) return FA8_ERR_SHAPE;
   if (p->heads_k < 0 || (p->heads_k > 0 && p->heads % p->heads_k != 0)) return FA8_ERR_SHAPE;
   if (p->causal_align != FA8_CAUSAL_TOP_LEFT && p->causal_align != FA8_CAUSAL_BOTTOM_RIGHT) return FA8_ERR_DTYPE;
+  if (p->schedule != FA8_SCHEDULE_AUTO && p->schedule != FA8_SCHEDULE_ROLLING && p->schedule != FA8_SCHEDULE_PIPELINED)
+    return FA8_ERR_DTYPE;
   if ((long long)p->batch * p->heads > 0x7fffffffLL / ((p->seqlen_q + kQBlock - 1) / kQBlock)) return FA8_ERR_SHAPE;
   if (p->in_dtype != FA8_DTYPE_E4M3 && p->in_dtype != FA8_DTYPE_E5M2) return FA8_ERR_DTYPE;
   if (p->out_dtype != FA8_OUT_FP16 && p->out_dtype != FA8_OUT_E4M3 && p->out_dtype != FA8_OUT_E5M2) return FA8_ERR_DTYPE;
@@ -687,9 +916,20 @@ extern "C" int fa8_fwd(const Fa8FwdParams* p, void* hip_stream) {
   a.v_bs = p->v_batch_stride; a.v_hs = p->v_head_stride; a.v_rs = p->v_row_stride;
   a.o_bs = p->o_batch_stride; a.o_hs = p->o_head_stride; a.o_rs = p->o_row_stride;
   hipStream_t stream = (hipStream_t)hip_stream;
+  // Which main loop (see fa8_fwd_kernel): the pipelined one up to four workgroups per compute unit (two resident at a
+  // time; measured 5 - 15 % faster there, also for the causal shapes whose workgroups thin out towards the end), the rolling
+  // one above (measured equal or up to 5 % faster).  The pipelined loop exists for head dims 64 and 128 and a positive
+  // softmax scale; elsewhere the hint is ignored.
+  bool pipelined = p->schedule == FA8_SCHEDULE_PIPELINED;
+  if (p->schedule == FA8_SCHEDULE_AUTO) {
+    const int cus = compute_units();
+    pipelined = cus > 0 && (long long)a.bh_total * a.n_qblocks <= 4LL * cus;
+  }
+  // the pipelined loop relies on exp2(-inf * scale) = 0 for masked logits
+  if (!(p->softmax_scale > 0.f)) pipelined = false;
   switch (p->head_dim) {
 #define FA8_HEAD_DIM_CASE(D_) \
-  case D_: return p->is_causal ? launch_types<D_, true>(p, a, stream) : launch_types<D_, false>(p, a, stream)
+  case D_: return p->is_causal ? launch_types<D_, true>(p, a, pipelined, stream) : launch_types<D_, false>(p, a, pipelined, stream)
     FA8_HEAD_DIM_CASE(32);  // the head-dim buckets of the reference (csrc/static_switch.h:50-77)
     FA8_HEAD_DIM_CASE(64);
     FA8_HEAD_DIM_CASE(96);

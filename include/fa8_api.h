@@ -38,6 +38,15 @@ extern "C" {
 #define FA8_CAUSAL_TOP_LEFT 0     /* key j <= query i: the reference's rule (csrc/flash_attention.cu:62-64, loop bound :458) */
 #define FA8_CAUSAL_BOTTOM_RIGHT 1 /* key j <= i + seqlen_k - seqlen_q: the last query sees every key (decode, chunked prefill) */
 
+/* which main loop the kernel runs: a performance hint, the results are bitwise the same
+ *   AUTO      the library chooses from the size of the launch
+ *   ROLLING   one KV block after the other, three wavefronts per SIMD: for launches that fill the chip
+ *   PIPELINED software-pipelined over neighbouring KV blocks, two wavefronts per SIMD: for small launches
+ *             (built for head dims 64 and 128; ignored for the others) */
+#define FA8_SCHEDULE_AUTO 0
+#define FA8_SCHEDULE_ROLLING 1
+#define FA8_SCHEDULE_PIPELINED 2
+
 /* error codes (all negative) */
 #define FA8_OK 0
 #define FA8_ERR_NULL (-1)        /* a required pointer is NULL */
@@ -45,7 +54,7 @@ extern "C" {
 #define FA8_ERR_HEAD_DIM (-3)    /* head_dim is not a multiple of 32 in 32..256 */
 #define FA8_ERR_STRIDE (-4)      /* a stride is smaller than the extent it must span, or rows overlap */
 #define FA8_ERR_ALIGN (-5)       /* a base pointer or stride breaks the 16-byte row alignment the kernels load with (FA8_V_TRANSPOSED: also seqlen_k % 16 != 0) */
-#define FA8_ERR_DTYPE (-6)       /* unknown in_dtype/out_dtype/v_layout/causal_align code */
+#define FA8_ERR_DTYPE (-6)       /* unknown in_dtype/out_dtype/v_layout/causal_align/schedule code */
 #define FA8_ERR_UNSUPPORTED (-7) /* a valid combination that this build has no kernel for */
 #define FA8_ERR_SCALE (-8)       /* softmax_scale is NaN or infinite */
 
@@ -87,6 +96,9 @@ typedef struct Fa8FwdParams {
    * declared, never used by its kernel.) */
   int32_t heads_k;
   int32_t causal_align; /* FA8_CAUSAL_* */
+  /* ---- library version 3; all-zero = the library chooses ---- */
+  int32_t schedule;  /* FA8_SCHEDULE_*: a performance hint, never changes the result */
+  int32_t reserved0; /* must be 0 */
 } Fa8FwdParams;
 
 /*
