@@ -301,14 +301,14 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PIPE ?
       (void*)vp, 0, VT ? (int)((D - 1) * a.v_rs + a.seqlen_k) : (int)(kv_last * a.v_rs + D), kRsrcFlags);
   // Start the asynchronous copy of the K rows / the V rows of KV block j into the LDS buffer kb / vb.
   auto issue_k = [&](int j, uint8_t* kb) __attribute__((always_inline)) {
-    const int k_base = j * kKvBlock * (int)a.k_rs;
+    const int k_base = (int)((unsigned)j * kKvBlock * (unsigned)a.k_rs);  // below 2^32 (fa8_fwd_validate)
 #pragma unroll
     for (int p = 0; p < kPasses; ++p)
       if (!kSplitPass || wave < 2)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, LDS_PTR(void, kb + copy_segment(p) * 1024), 16, k_src[p], k_base, 0, 0);
   };
   auto issue_v = [&](int j, uint8_t* vb) __attribute__((always_inline)) {
-    const int v_base = VT ? j * kKvBlock : j * kKvBlock * (int)a.v_rs;
+    const int v_base = VT ? j * kKvBlock : (int)((unsigned)j * kKvBlock * (unsigned)a.v_rs);
     // transposed v, ragged last block: the 16-byte chunks past the last kv column would read the start of the next
     // head-dim row (or run off the tensor); they are pulled back onto the last chunk instead (and masked later)
     const bool v_clamp = VT && (j + 1) * kKvBlock > a.seqlen_k;
@@ -622,11 +622,11 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PIPE ?
     using F = std::false_type;
     // the copies of steps -4 .. -1
     issue_k(0, k_lds0);
-    issue_k(1, k_lds1);
-    issue_k(2, k_lds2);
+    issue_k(min(1, n_tiles), k_lds1);
+    issue_k(min(2, n_tiles), k_lds2);
     issue_v(0, v_lds0);
-    issue_k(3, k_lds3);
-    issue_v(1, v_lds1);
+    issue_k(min(3, n_tiles), k_lds3);
+    issue_v(min(1, n_tiles), v_lds1);
     wait_in_flight(std::integral_constant<int, 5>());  // K(0) landed
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
@@ -642,8 +642,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PIPE ?
       constexpr bool kFirst = decltype(first_c)::value;
       uint8_t* const kst[4] = {k_lds0, k_lds1, k_lds2, k_lds3};
       uint8_t* const vst[4] = {v_lds0, v_lds1, v_lds2, v_lds3};
-      issue_k(j + 4, kst[PH]);
-      issue_v(j + 2, vst[(PH + 2) % 4]);
+      issue_k(min(j + 4, n_tiles), kst[PH]);  // (block n_tiles lies wholly beyond the buffer)
+      issue_v(min(j + 2, n_tiles), vst[(PH + 2) % 4]);
       iteration(first_c, j, kst[(PH + 1) % 4], vst[(PH + 3) % 4], sbuf[PH % 2], sbuf[(PH + 1) % 2], p8buf[(PH + 1) % 2],
                 p8buf[PH % 2]);
       end_step();
@@ -884,6 +884,11 @@ extern "C" int fa8_fwd_validate(const Fa8FwdParams* p) {
   const long long k_rows_addr = p->seqlen_k > kKvBlock ? p->seqlen_k : kKvBlock;
   const long long v_rows_addr = v_rows > kKvBlock ? v_rows : kKvBlock;
   if (k_rows_addr * p->k_row_stride > 0x7fffffffLL || v_rows_addr * p->v_row_stride > 0x7fffffffLL) return FA8_ERR_SHAPE;
+  // ... and the offsets of a whole block just past the last row (block offset + row offset of its 64th row) must not wrap
+  // around 32 bits, or the buffer's range check would take them for rows of the tensor (matters only for a few rows with a
+  // row stride of tens of megabytes)
+  if ((p->seqlen_k + 126LL) * p->k_row_stride + 256 > 0xffffffffLL || (v_rows + 126LL) * p->v_row_stride + 256 > 0xffffffffLL)
+    return FA8_ERR_SHAPE;
   // transposed v is read in 16-byte chunks along kv
   if (p->v_layout == FA8_V_TRANSPOSED && p->seqlen_k % 16 != 0) return FA8_ERR_ALIGN;
   // an fp8 output has the element type of the inputs
