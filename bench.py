@@ -127,8 +127,8 @@ def main():
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py: this build runs on one GPU only (the path shards over batch*heads with no communication; "
-              "see DESIGN.md); run with --gpus 1", file=sys.stderr)
+        print("bench.py: this build runs on one GPU only (every (batch, head) is independent: more GPUs would each take a "
+              "range of heads and run this same kernel, with no communication); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
 
     if args.instruction_mix:
