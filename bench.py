@@ -10,6 +10,7 @@ cores of the same machine on a bounded sample of heads).
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3] [--no-cpu-baseline]
 """
 import argparse
+import ctypes
 import json
 import os
 import sys
@@ -166,6 +167,9 @@ def main():
     def step():
         return ext.flash_attention_v2_cutlass(q, k, v, causal, scale)[0]
 
+    # which of the kernel's two main loops the library runs for this launch (include/fa8_api.h, FA8_SCHEDULE_*)
+    plan = fa.lib().fa8_fwd_schedule(ctypes.byref(fa.make_params(q, k, v, step(), causal, scale)))
+    main_loop = {fa.FA8_SCHEDULE_ROLLING: "rolling", fa.FA8_SCHEDULE_PIPELINED: "pipelined"}.get(plan, f"error {plan}")
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -231,6 +235,7 @@ def main():
             "pct_fp8_mfma_peak": round(100.0 * tflops / FP8_MFMA_PEAK_TFLOPS, 2),
             "algorithmic_hbm_gbps": round(alg_bytes / (kern_avg_ms * 1e-3) / 1e9, 1),
             "kv_block": fa.query(fa.FA8_QUERY_KV_BLOCK),
+            "main_loop": main_loop,
             "sclk_mhz_under_load": sclk,
             "settle_launches": settle_launches,
         },

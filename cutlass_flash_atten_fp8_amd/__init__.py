@@ -29,7 +29,7 @@ FA8_CAUSAL_TOP_LEFT, FA8_CAUSAL_BOTTOM_RIGHT = 0, 1
 FA8_SCHEDULE_AUTO, FA8_SCHEDULE_ROLLING, FA8_SCHEDULE_PIPELINED = 0, 1, 2
 (FA8_QUERY_VERSION, FA8_QUERY_KV_BLOCK, FA8_QUERY_Q_BLOCK, FA8_QUERY_KV_ASCENDING, FA8_QUERY_THREADS,
  FA8_QUERY_PARAMS_SIZE) = range(6)
-FA8_EXPORTS = ("fa8_fwd_validate", "fa8_fwd", "fa8_query", "fa8_error_string")
+FA8_EXPORTS = ("fa8_fwd_validate", "fa8_fwd", "fa8_fwd_schedule", "fa8_query", "fa8_error_string")
 
 
 class Fa8FwdParams(ctypes.Structure):
@@ -66,6 +66,8 @@ def lib():
         L.fa8_fwd_validate.argtypes = [ctypes.POINTER(Fa8FwdParams)]
         L.fa8_fwd.restype = ctypes.c_int
         L.fa8_fwd.argtypes = [ctypes.POINTER(Fa8FwdParams), ctypes.c_void_p]
+        L.fa8_fwd_schedule.restype = ctypes.c_int
+        L.fa8_fwd_schedule.argtypes = [ctypes.POINTER(Fa8FwdParams)]
         L.fa8_query.restype = ctypes.c_int
         L.fa8_query.argtypes = [ctypes.c_int]
         L.fa8_error_string.restype = ctypes.c_char_p

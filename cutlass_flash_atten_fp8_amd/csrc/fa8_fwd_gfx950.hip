@@ -826,20 +826,21 @@ int launch_types(const Fa8FwdParams* p, const KernelArgs& a, bool pipelined, hip
   return p->out_dtype == FA8_OUT_E4M3 ? launch<D, CAUSAL, false, FA8_OUT_E4M3>(a, vt, pipelined, stream) : FA8_ERR_UNSUPPORTED;
 }
 
-// KV blocks walked by all workgroups of a launch together (causal: approximated to within a block per workgroup).
-long long launch_kv_blocks(const Fa8FwdParams* p, const KernelArgs& a) {
-  const long long nq = a.n_qblocks, tk = (p->seqlen_k + kKvBlock - 1) / kKvBlock;
-  if (!p->is_causal) return (long long)a.bh_total * nq * tk;
+// KV blocks walked by all workgroups of a launch together.
+long long launch_kv_blocks(const Fa8FwdParams* p) {
+  const long long bh = (long long)p->batch * p->heads, nq = (p->seqlen_q + kQBlock - 1) / kQBlock;
+  const long long tk = (p->seqlen_k + kKvBlock - 1) / kKvBlock;
+  if (!p->is_causal) return bh * nq * tk;
   // q block i walks clamp(base + 2 i, 1, tk) blocks: one block up to i = n1 - 1, all tk blocks from i = first
-  const long long s64 = a.causal_shift, base = 2 + (s64 >= 0 ? (s64 + kKvBlock - 1) / kKvBlock : -((-s64) / kKvBlock));
+  const long long s64 = p->causal_align == FA8_CAUSAL_BOTTOM_RIGHT ? (long long)p->seqlen_k - p->seqlen_q : 0;
+  const long long base = 2 + (s64 >= 0 ? (s64 + kKvBlock - 1) / kKvBlock : -((-s64) / kKvBlock));
   long long n1 = base <= 1 ? (1 - base) / 2 + 1 : 0;
   if (n1 > nq) n1 = nq;
   long long first = tk > base ? (tk - base + 1) / 2 : 0;
   if (first < n1) first = n1;
   if (first > nq) first = nq;
   const long long cnt = first - n1;
-  const long long per_head = n1 + cnt * base + (n1 + first - 1) * cnt + (nq - first) * tk;
-  return (long long)a.bh_total * per_head;
+  return bh * (n1 + cnt * base + (n1 + first - 1) * cnt + (nq - first) * tk);
 }
 
 // Compute units of the current device (0 if the runtime cannot tell), asked once per device.
@@ -853,6 +854,23 @@ int compute_units() {
     cached[dev] = n;
   }
   return cached[dev];
+}
+
+// Which main loop a valid call runs (see fa8_fwd_kernel).  The pipelined one for launches that cannot keep three wavefronts on
+// every SIMD for most of their run: at most four workgroups per compute unit (two resident at a time), or little work per
+// compute unit (then filling and draining the chip, and for causal launches the thinning out of the workgroups, is a large
+// share of the run).  Measured 5 - 15 % faster there; the rolling loop is equal or up to 5 % faster elsewhere.  The pipelined
+// loop exists for head dims 64 and 128 and relies on exp2(-inf * scale) = 0 for masked logits, i.e. on a positive softmax
+// scale; elsewhere the hint is ignored.
+bool runs_pipelined(const Fa8FwdParams* p) {
+  if ((p->head_dim != 64 && p->head_dim != 128) || !(p->softmax_scale > 0.f)) return false;
+  if (p->schedule != FA8_SCHEDULE_AUTO) return p->schedule == FA8_SCHEDULE_PIPELINED;
+  const long long cus = compute_units();
+  const long long wgs = (long long)p->batch * p->heads * ((p->seqlen_q + kQBlock - 1) / kQBlock);
+  // KV blocks per compute unit below which the pipelined loop was measured to win (head dim 64 has half the matrix work
+  // per block)
+  const long long few_blocks = p->head_dim == 64 ? 264 : 144;
+  return cus > 0 && (wgs <= 4 * cus || (wgs <= few_blocks * cus && launch_kv_blocks(p) <= few_blocks * cus));
 }
 
 bool span_ok(long long outer_stride, long long inner_extent) { return outer_stride >= inner_extent; }
@@ -937,22 +955,7 @@ extern "C" int fa8_fwd(const Fa8FwdParams* p, void* hip_stream) {
   a.v_bs = p->v_batch_stride; a.v_hs = p->v_head_stride; a.v_rs = p->v_row_stride;
   a.o_bs = p->o_batch_stride; a.o_hs = p->o_head_stride; a.o_rs = p->o_row_stride;
   hipStream_t stream = (hipStream_t)hip_stream;
-  // Which main loop (see fa8_fwd_kernel).  The pipelined one for launches that cannot keep three wavefronts on every SIMD
-  // for most of their run: at most four workgroups per compute unit (two resident at a time), or little work per compute
-  // unit (then filling and draining the chip, and for causal launches the thinning out of the workgroups, is a large share
-  // of the run).  Measured 5 - 15 % faster there; the rolling loop is equal or up to 5 % faster elsewhere.  The pipelined loop
-  // exists for head dims 64 and 128 and a positive softmax scale; elsewhere the hint is ignored.
-  bool pipelined = p->schedule == FA8_SCHEDULE_PIPELINED;
-  if (p->schedule == FA8_SCHEDULE_AUTO) {
-    const long long cus = compute_units();
-    const long long wgs = (long long)a.bh_total * a.n_qblocks;
-    // KV blocks per compute unit below which the pipelined loop was measured to win (head dim 64 has half the matrix work
-    // per block)
-    const long long few_blocks = p->head_dim <= 64 ? 264 : 144;
-    pipelined = cus > 0 && (wgs <= 4 * cus || (wgs <= few_blocks * cus && launch_kv_blocks(p, a) <= few_blocks * cus));
-  }
-  // the pipelined loop relies on exp2(-inf * scale) = 0 for masked logits
-  if (!(p->softmax_scale > 0.f)) pipelined = false;
+  const bool pipelined = runs_pipelined(p);
   switch (p->head_dim) {
 #define FA8_HEAD_DIM_CASE(D_) \
   case D_: return p->is_causal ? launch_types<D_, true>(p, a, pipelined, stream) : launch_types<D_, false>(p, a, pipelined, stream)
@@ -967,6 +970,12 @@ extern "C" int fa8_fwd(const Fa8FwdParams* p, void* hip_stream) {
 #undef FA8_HEAD_DIM_CASE
     default: return FA8_ERR_HEAD_DIM;
   }
+}
+
+extern "C" int fa8_fwd_schedule(const Fa8FwdParams* p) {
+  const int rc = fa8_fwd_validate(p);
+  if (rc != FA8_OK) return rc;
+  return runs_pipelined(p) ? FA8_SCHEDULE_PIPELINED : FA8_SCHEDULE_ROLLING;
 }
 
 extern "C" int fa8_query(int what) {

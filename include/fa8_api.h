@@ -116,6 +116,14 @@ int fa8_fwd_validate(const Fa8FwdParams* p);
  */
 int fa8_fwd(const Fa8FwdParams* p, void* hip_stream);
 
+/*
+ * Which main loop fa8_fwd would run for these arguments on the current device: FA8_SCHEDULE_ROLLING or
+ * FA8_SCHEDULE_PIPELINED (both > 0), or the FA8_ERR_* code fa8_fwd_validate gives.  Launches nothing.  No counterpart in
+ * the reference (one kernel, one loop: csrc/flash_attention.cu:468-534); it makes the library's choice visible to
+ * benchmarks and tests.
+ */
+int fa8_fwd_schedule(const Fa8FwdParams* p);
+
 /* What fa8_query can report. */
 #define FA8_QUERY_VERSION 0       /* integer library version */
 #define FA8_QUERY_KV_BLOCK 1      /* kv columns per online-softmax step (reference kBlockN = 64, csrc/flash_attention.cu:624) */

@@ -141,3 +141,22 @@ def test_compiled_binding_mirrors_reference_errors():
     with pytest.raises(TypeError):
         ext.flash_attention_v2_cutlass(q, k, v)
     assert ext.kv_block() == fa.query(fa.FA8_QUERY_KV_BLOCK)
+
+
+def test_schedule_query_follows_explicit_hints_without_a_gpu():
+    """fa8_fwd_schedule: an explicit hint is answered without touching the GPU; it holds only where the pipelined loop exists."""
+    sched = fa.lib().fa8_fwd_schedule
+    for d, scale, hint, want in ((128, 0.1, fa.FA8_SCHEDULE_PIPELINED, fa.FA8_SCHEDULE_PIPELINED),
+                                 (64, 0.1, fa.FA8_SCHEDULE_PIPELINED, fa.FA8_SCHEDULE_PIPELINED),
+                                 (128, 0.1, fa.FA8_SCHEDULE_ROLLING, fa.FA8_SCHEDULE_ROLLING),
+                                 (96, 0.1, fa.FA8_SCHEDULE_PIPELINED, fa.FA8_SCHEDULE_ROLLING),
+                                 (256, 0.1, fa.FA8_SCHEDULE_AUTO, fa.FA8_SCHEDULE_ROLLING),
+                                 (128, -0.1, fa.FA8_SCHEDULE_PIPELINED, fa.FA8_SCHEDULE_ROLLING),
+                                 (64, 0.0, fa.FA8_SCHEDULE_AUTO, fa.FA8_SCHEDULE_ROLLING)):
+        q, k, v, o = cpu_tensors(d=d)
+        p = fa.make_params(q, k, v, o, True, scale, schedule=hint)
+        assert sched(ctypes.byref(p)) == want, (d, scale, hint)
+    q, k, v, o = cpu_tensors()
+    p = fa.make_params(q, k, v, o, False, 0.1, schedule=9)
+    assert sched(ctypes.byref(p)) == -6 and validate(p) == -6  # FA8_ERR_DTYPE: unknown schedule code
+    assert sched(None) == -1

@@ -85,3 +85,20 @@ def test_non_positive_scale_and_other_head_dims_ignore_the_hint():
         assert torch.equal(a.view(torch.int16), b.view(torch.int16))
     with pytest.raises(RuntimeError):
         fa.flash_attention_v2_cutlass(q.to(DEV), k.to(DEV), v.to(DEV), True, 0.1, schedule=7)
+
+
+def test_library_choice_by_launch_size():
+    """fa8_fwd_schedule on the GPU box: small launches take the pipelined loop, launches that fill the chip the rolling one."""
+    import ctypes
+
+    def plan(B, H, N, d, causal):
+        q = torch.empty((B, H, N, d), dtype=torch.float8_e4m3fn, device=DEV)
+        o = torch.empty((B, H, N, d), dtype=torch.float16, device=DEV)
+        return fa.lib().fa8_fwd_schedule(ctypes.byref(fa.make_params(q, q, q, o, causal, d ** -0.5)))
+
+    assert plan(1, 16, 1024, 128, True) == fa.FA8_SCHEDULE_PIPELINED      # 128 workgroups
+    assert plan(4, 16, 1024, 64, False) == fa.FA8_SCHEDULE_PIPELINED      # 512 workgroups (cfg2)
+    assert plan(4, 32, 2048, 64, True) == fa.FA8_SCHEDULE_PIPELINED       # 2048 short causal workgroups: little work per CU
+    assert plan(2, 32, 4096, 128, False) == fa.FA8_SCHEDULE_ROLLING       # the headline shape
+    assert plan(1, 32, 8192, 128, True) == fa.FA8_SCHEDULE_ROLLING        # cfg4
+    assert plan(1, 16, 1024, 96, True) == fa.FA8_SCHEDULE_ROLLING         # no pipelined loop for this head dim
