@@ -105,6 +105,25 @@ def read_sclk_mhz():
     return None
 
 
+def read_power_w():
+    """(board power now, power cap) in watts from the amdgpu hwmon node, None where a file is missing."""
+    import glob
+
+    def first(pattern):
+        for path in sorted(glob.glob(pattern)):
+            try:
+                with open(path) as f:
+                    return int(f.read().strip()) / 1e6
+            except (OSError, ValueError):
+                pass
+        return None
+    base = "/sys/class/drm/card*/device/hwmon/hwmon*/"
+    now = first(base + "power1_average")
+    if now is None:
+        now = first(base + "power1_input")
+    return now, first(base + "power1_cap")
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -200,15 +219,19 @@ def main():
     # shader clock while the kernel is running (power management lowers it under dense matrix work): sampled in the
     # middle of untimed bursts of launches long enough to keep the queue full whatever --steps is, median of 16 readings
     burst = max(25, int(0.008 / max(kern_ms[len(kern_ms) // 2] * 1e-3, 1e-6)))  # about 8 ms of kernel time per burst
-    samples = []
+    samples, watts = [], []
     for _ in range(20):
         for _ in range(burst):
             step()
         time.sleep(0.004)  # the queue stays full: the launches above take about twice as long as this
         samples.append(read_sclk_mhz())
+        watts.append(read_power_w()[0])
     torch.cuda.synchronize()
     samples = sorted(x for x in samples[4:] if x is not None)
     sclk = samples[len(samples) // 2] if samples else None
+    watts = sorted(x for x in watts[4:] if x is not None)
+    power_w = round(watts[len(watts) // 2]) if watts else None
+    power_cap_w = read_power_w()[1]
     kern_avg_ms = sum(kern_ms) / len(kern_ms)
 
     tflops = flops / (wall_ms * 1e-3) / 1e12
@@ -237,6 +260,8 @@ def main():
             "kv_block": fa.query(fa.FA8_QUERY_KV_BLOCK),
             "main_loop": main_loop,
             "sclk_mhz_under_load": sclk,
+            "board_power_w_under_load": power_w,
+            "board_power_cap_w": round(power_cap_w) if power_cap_w is not None else None,
             "settle_launches": settle_launches,
         },
         "roofline": {
