@@ -40,6 +40,9 @@ CASES = [
     (1, 3, 3, 130, 1500, 128, False, False, False, torch.float8_e4m3fn, torch.float16),
     (1, 2, 2, 2048, 2048, 128, True, False, False, torch.float8_e4m3fn, torch.float16),
     (1, 8, 8, 1024, 1024, 64, False, False, False, torch.float8_e4m3fn, torch.float16),
+    (2, 32, 32, 4096, 4096, 128, False, False, False, torch.float8_e4m3fn, torch.float16),  # the headline shape
+    (1, 8, 8, 8192, 8192, 128, True, False, False, torch.float8_e4m3fn, torch.float16),
+    (1, 16, 4, 4160, 4160, 64, True, False, False, torch.float8_e4m3fn, torch.float16),
 ]
 
 
