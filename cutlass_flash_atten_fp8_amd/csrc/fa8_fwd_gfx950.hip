@@ -587,7 +587,11 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PIPE ?
         sum1 = (u == 0) ? s[t][4 * w + 1] : sum1 + s[t][4 * w + 1];
         sum0 += s[t][4 * w + 2];
         sum1 += s[t][4 * w + 3];
-        p8_cur[u] = pack4_fp8<E5M2>(s[t][4 * w], s[t][4 * w + 1], s[t][4 * w + 2], s[t][4 * w + 3]);
+        int packed = pack4_fp8<E5M2>(s[t][4 * w], s[t][4 * w + 1], s[t][4 * w + 2], s[t][4 * w + 3]);
+        // the weights are only read in the next iteration; without this pin the compiler sinks the conversions there, in
+        // one clump in front of the PV products that wait for them
+        asm volatile("" : "+v"(packed));
+        p8_cur[u] = packed;
         __builtin_amdgcn_sched_barrier(0);
       }
       l_run += sum0 + sum1;
