@@ -91,3 +91,20 @@ def test_large_configs_sampled(name):
     cfg = inputs.CONFIGS[name]
     q, k, v = inputs.make_qkv(cfg)
     check(q, k, v, inputs.softmax_scale(cfg), cfg["causal"], rows=sample_rows(cfg["N"], 512), label=name)
+
+
+@pytest.mark.parametrize("B,H,N,d", [(1, 88, 300, 64), (3, 24, 200, 128), (1, 12, 260, 64), (1, 40, 140, 96), (2, 8, 520, 128)])
+@pytest.mark.parametrize("causal", [False, True])
+def test_every_head_and_q_block_is_computed(B, H, N, d, causal):
+    """Workgroup ids are mapped to (head, q block) differently for full and causal launches, for head counts that are and are
+    not multiples of the 8 XCDs, and in groups of up to 8 heads per XCD (88 heads: one group of 8 and one of 3; 72: 8 and 1):
+    a hole or a double in that map would leave rows of some head unwritten.  The output starts as NaN."""
+    g = torch.Generator().manual_seed(B * 1000 + H)
+    q, k, v = (torch.randn((B, H, N, d), generator=g).to(torch.float8_e4m3fn) for _ in range(3))
+    dev = torch.device("cuda:0")
+    o = torch.full((B, H, N, d), float("nan"), dtype=torch.float16, device=dev)
+    run_abi(q.to(dev), k.to(dev), v.to(dev), causal, d ** -0.5, o=o)
+    assert torch.isfinite(o).all()
+    rows = sample_rows(N, 24, seed=H)
+    assert_parity(o.float().cpu().numpy()[:, :, rows, :], u8(q), u8(k), u8(v), d ** -0.5, causal=causal, rows=rows,
+                  kv_block=fa.query(fa.FA8_QUERY_KV_BLOCK), label=f"map B{B} H{H} N{N} d{d} causal={causal}")
