@@ -188,7 +188,7 @@ def main():
 
     # which of the kernel's two main loops the library runs for this launch (include/fa8_api.h, FA8_SCHEDULE_*)
     plan = fa.lib().fa8_fwd_schedule(ctypes.byref(fa.make_params(q, k, v, step(), causal, scale)))
-    main_loop = {fa.FA8_SCHEDULE_ROLLING: "rolling", fa.FA8_SCHEDULE_PIPELINED: "pipelined"}.get(plan, f"error {plan}")
+    main_loop = {fa.FA8_SCHEDULE_ROLLING: "rolling", fa.FA8_SCHEDULE_PIPELINED: "pipelined", fa.FA8_SCHEDULE_DENSE: "dense"}.get(plan, f"error {plan}")
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()

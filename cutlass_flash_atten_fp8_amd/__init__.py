@@ -26,7 +26,7 @@ FA8_DTYPE_E4M3, FA8_DTYPE_E5M2 = 0, 1
 FA8_OUT_FP16, FA8_OUT_E4M3, FA8_OUT_E5M2 = 0, 1, 2
 FA8_V_ROWS, FA8_V_TRANSPOSED = 0, 1
 FA8_CAUSAL_TOP_LEFT, FA8_CAUSAL_BOTTOM_RIGHT = 0, 1
-FA8_SCHEDULE_AUTO, FA8_SCHEDULE_ROLLING, FA8_SCHEDULE_PIPELINED = 0, 1, 2
+FA8_SCHEDULE_AUTO, FA8_SCHEDULE_ROLLING, FA8_SCHEDULE_PIPELINED, FA8_SCHEDULE_DENSE = 0, 1, 2, 3
 (FA8_QUERY_VERSION, FA8_QUERY_KV_BLOCK, FA8_QUERY_Q_BLOCK, FA8_QUERY_KV_ASCENDING, FA8_QUERY_THREADS,
  FA8_QUERY_PARAMS_SIZE) = range(6)
 FA8_EXPORTS = ("fa8_fwd_validate", "fa8_fwd", "fa8_fwd_schedule", "fa8_query", "fa8_error_string")

@@ -87,6 +87,8 @@ std::vector<torch::Tensor> flash_attention_v2_cutlass(torch::Tensor q, torch::Te
   p.o_batch_stride = out.stride(0); p.o_head_stride = out.stride(1); p.o_row_stride = out.stride(2);
   p.heads_k = (int32_t)Hk;
   p.causal_align = causal_bottom_right ? FA8_CAUSAL_BOTTOM_RIGHT : FA8_CAUSAL_TOP_LEFT;
+  TORCH_CHECK(schedule >= FA8_SCHEDULE_AUTO && schedule <= FA8_SCHEDULE_DENSE, "schedule must be one of the FA8_SCHEDULE_* codes 0..",
+              FA8_SCHEDULE_DENSE, ", got ", schedule);
   p.schedule = (int32_t)schedule;
   if (return_lse) {
     p.lse = lse.data_ptr();

@@ -23,6 +23,7 @@
 //     the swizzle being applied on the global-address side of the copy.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cmath>
 #include <cstdint>
 #include <type_traits>
@@ -30,8 +31,8 @@
 #include "fa8_api.h"
 
 // wavefronts per SIMD the kernels are compiled for: 3 (at most 168 VGPRs per lane) up to head dim 128, 2 (256 VGPRs:
-// the output accumulators alone take 128) for head dim 256
-#define FA8_WAVES_PER_EU(D) ((D) > 128 ? 2 : 3)
+// the output accumulators alone take 128) for head dim 256; the pipelined loop 2; the dense loop 3 (head dim 64: 4)
+#define FA8_WAVES_PER_EU(D, LOOP) ((LOOP) == 1 ? 2 : ((LOOP) == 2 ? ((D) == 64 ? 4 : 3) : ((D) > 128 ? 2 : 3)))
 
 namespace {
 
@@ -48,7 +49,9 @@ constexpr int kQBlock = 128;   // query rows per workgroup
 constexpr int kQWave = 32;     // query rows per wavefront
 constexpr int kKvBlock = 64;   // kv rows per online-softmax step
 constexpr int kThreads = 256;  // 4 wavefronts
-constexpr int kVersion = 3;
+constexpr int kVersion = 4;
+// main loops (template parameter LOOP of the kernel)
+constexpr int kLoopRolling = 0, kLoopPipelined = 1, kLoopDense = 2;
 
 struct KernelArgs {
   const uint8_t* q;
@@ -200,17 +203,23 @@ __device__ __forceinline__ void decode_block(const KernelArgs& a, int id, int& b
   qb = CAUSAL ? (a.n_qblocks - 1 - qi) : qi;
 }
 
-// PIPE selects the main loop.  false: one KV block after the other (S^T, softmax, PV), three wavefronts per SIMD hide each
-// other's latencies: the loop for launches that fill the chip.  true: a software-pipelined loop for launches that leave
-// a SIMD with two wavefronts or fewer (short sequences, few heads): the matrix instructions of the neighbouring blocks
-// (PV of block j-1, S^T of block j+1) are issued between the chunks of the softmax of block j, so that one wavefront alone
-// keeps the matrix and the vector pipe busy; it needs about 200 VGPRs (two wavefronts per SIMD) and four LDS stages.
-// Both loops perform the same arithmetic in the same order: their results are bitwise equal.
-template <int D, bool CAUSAL, bool E5M2, int OUT, bool VT, bool PIPE>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PIPE ? 2 : FA8_WAVES_PER_EU(D)))) void fa8_fwd_kernel(
+// LOOP selects the main loop; all three perform the same arithmetic in the same order, their results are bitwise equal.
+// kLoopRolling: one KV block after the other (S^T, softmax, PV), three wavefronts per SIMD hide each other's latencies.
+// kLoopPipelined: software-pipelined for launches that leave a SIMD with two wavefronts or fewer (short sequences, few
+// heads): the matrix instructions of the neighbouring blocks (PV of block j-1, S^T of block j+1) are issued between the
+// chunks of the softmax of block j, so that one wavefront alone keeps the matrix and the vector pipe busy; about 180
+// VGPRs (two wavefronts per SIMD), four LDS stages; every block may be masked.
+// kLoopDense: the same pipeline squeezed into 168 VGPRs (three wavefronts per SIMD, three LDS stages) for launches
+// in which no block needs a mask (full attention over a whole number of KV blocks): one logits buffer, whose halves are
+// refilled by the S^T products of block j+1 as soon as the softmax of block j has turned them into weights.
+template <int D, bool CAUSAL, bool E5M2, int OUT, bool VT, int LOOP>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WAVES_PER_EU(D, LOOP)))) void fa8_fwd_kernel(
     const KernelArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the body uses device-only types (buffer resources); the host pass only needs the stub
   static_assert(D % 32 == 0 && D >= 32 && D <= 256, "head dims: multiples of 32 up to 256");
+  constexpr bool PIPE = LOOP == kLoopPipelined, DENSE = LOOP == kLoopDense;
+  static_assert(LOOP == kLoopRolling || D == 64 || D == 128, "the pipelined loops are built for head dims 64 and 128");
+  static_assert(!DENSE || !CAUSAL, "the dense loop has no masks");
   // LDS tiles are laid out for the next power of two: rows of DP bytes, of which the first D are used
   constexpr int DP = D <= 32 ? 32 : (D <= 64 ? 64 : (D <= 128 ? 128 : 256));
   constexpr int kTileBytes = kKvBlock * DP;  // one K or V tile
@@ -222,7 +231,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PIPE ?
   constexpr int kMTiles = D / 32;         // 32-row tiles of O^T
   // LDS stages per operand: three (copies issued two KV blocks ahead) where three workgroups then still fit in the
   // 160 KB of a CU, two for head dims above 128 (2 x 32 KB per workgroup, two workgroups per CU)
-  // (the pipelined loop: four, copies issued up to four blocks ahead)
+  // (the pipelined loop: four, copies issued up to four blocks ahead; the dense loop: three)
   constexpr int kStages = PIPE ? 4 : (D > 128 ? 2 : 3);
   // One LDS object per (stage, operand): the compiler then knows that the asynchronous HBM -> LDS copy into one
   // stage cannot alias the reads of the other stage and does not wait for the copy before those reads.
@@ -295,19 +304,25 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PIPE ?
   }
   const int kv_last = a.seqlen_k - 1;
   constexpr int kRsrcFlags = 0x00020000;  // raw buffer, 32-bit data format
-  const __amdgpu_buffer_rsrc_t k_rsrc =
-      __builtin_amdgcn_make_buffer_rsrc((void*)kp, 0, (int)(kv_last * a.k_rs + D), kRsrcFlags);
-  const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)vp, 0, VT ? (int)((D - 1) * a.v_rs + a.seqlen_k) : (int)(kv_last * a.v_rs + D), kRsrcFlags);
-  // Start the asynchronous copy of the K rows / the V rows of KV block j into the LDS buffer kb / vb.
-  auto issue_k = [&](int j, uint8_t* kb) __attribute__((always_inline)) {
+  // Start the asynchronous copy of the K rows / the V rows of KV block j into the LDS buffer kb / vb.  The pipelined loops
+  // start two tile copies in every step, also when the block no longer exists (so that one s_waitcnt constant fits every
+  // step): such a copy (exists = false, wave-uniform) goes through a resource of length 0, every lane of it is out of range,
+  // zeros land in LDS and no memory is touched.
+  // (Dense loop: the second pass of a copy differs from the first by a whole number of rows, 16 kv rows of K and 32 (64) rows
+  // of V (V^T): the difference sits in the scalar offset and both passes share one vector register.)
+  const int k_bytes = (int)(kv_last * a.k_rs + D);
+  const int v_bytes = VT ? (int)((D - 1) * a.v_rs + a.seqlen_k) : (int)(kv_last * a.v_rs + D);
+  auto issue_k = [&](int j, uint8_t* kb, bool exists) __attribute__((always_inline)) {
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)kp, 0, exists ? k_bytes : 0, kRsrcFlags);
     const int k_base = (int)((unsigned)j * kKvBlock * (unsigned)a.k_rs);  // below 2^32 (fa8_fwd_validate)
 #pragma unroll
     for (int p = 0; p < kPasses; ++p)
       if (!kSplitPass || wave < 2)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, LDS_PTR(void, kb + copy_segment(p) * 1024), 16, k_src[p], k_base, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, LDS_PTR(void, kb + copy_segment(p) * 1024), 16, DENSE ? k_src[0] : k_src[p],
+                                                 DENSE ? k_base + p * 16 * (int)a.k_rs : k_base, 0, 0);
   };
-  auto issue_v = [&](int j, uint8_t* vb) __attribute__((always_inline)) {
+  auto issue_v = [&](int j, uint8_t* vb, bool exists) __attribute__((always_inline)) {
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)vp, 0, exists ? v_bytes : 0, kRsrcFlags);
     const int v_base = VT ? j * kKvBlock : (int)((unsigned)j * kKvBlock * (unsigned)a.v_rs);
     // transposed v, ragged last block: the 16-byte chunks past the last kv column would read the start of the next
     // head-dim row (or run off the tensor); they are pulled back onto the last chunk instead (and masked later)
@@ -320,16 +335,17 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PIPE ?
           int r, ch;
           tile_slot_decode<64, false>(copy_segment(p) * 64 + lane, r, ch);
           const unsigned off = r < D ? (unsigned)(r * (int)a.v_rs + min(v_base + ch * 16, a.seqlen_k - 16)) : kNoSource;
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(v_rsrc, LDS_PTR(void, vb + seg), 16, off, 0, 0, 0);
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, LDS_PTR(void, vb + seg), 16, off, 0, 0, 0);
         } else {
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(v_rsrc, LDS_PTR(void, vb + seg), 16, v_src[p], v_base, 0, 0);
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, LDS_PTR(void, vb + seg), 16, DENSE ? v_src[0] : v_src[p],
+                                                   DENSE ? v_base + p * (VT ? 64 : 32) * (int)a.v_rs : v_base, 0, 0);
         }
       }
     }
   };
   auto issue_tile = [&](int j, uint8_t* kb, uint8_t* vb) __attribute__((always_inline)) {
-    issue_k(j, kb);
-    issue_v(j, vb);
+    issue_k(j, kb, true);
+    issue_v(j, vb, true);
   };
 
   // ---- per-lane LDS read offsets ----
@@ -493,7 +509,170 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PIPE ?
   };
   static_assert(kLoadsPerTile < 16, "vmcnt immediate above");
 
-  if constexpr (PIPE) {
+  if constexpr (DENSE) {
+    // ---- dense loop: the software pipeline in 168 VGPRs ----
+    // Iteration j is the softmax of block j in 8 chunks of 4 weights.  In front of chunks 0-3 go the PV products of block j-1
+    // (head dim 64: chunks 0 and 2), in front of chunks 4-5 the S^T products of sub-tile 0 of block j+1, written over sub-tile 0
+    // of block j, which is all weights by then; the S^T products of sub-tile 1 follow the last chunk and run under the rescale
+    // of O.  LDS operands are fetched one matrix instruction ahead.  K(t) and V(t) live in stage t % 3.  Step j starts the
+    // copies of K(j+3) (its stage held K(j), last read in step j-1) and V(j+1) (its stage held V(j-2), last read in step j-1)
+    // in front of chunks 1 and 2, reads K(j+1) and V(j-1), and ends when K(j+2) and V(j), started in step j-1, have landed.
+    v16f s[2];
+    v8i p8;
+    constexpr int kPvEvery = 4 / kMTiles;  // the PV product of tile mt goes in front of chunk mt * kPvEvery
+    constexpr int kSEvery = 2 / kKSteps;   // the S^T product (sub-tile 0, k-step ks) in front of chunk 4 + ks * kSEvery
+    auto iteration = [&](auto first_c, int j, const uint8_t* kb_next, const uint8_t* vb_prev, uint8_t* k_dst, uint8_t* v_dst)
+                         __attribute__((always_inline)) {
+      constexpr bool kFirst = decltype(first_c)::value;
+      v8i vfrag[kMTiles];
+      v8i kfrag[2][kKSteps];
+      if constexpr (!kFirst) vfrag[0] = load_vf(vb_prev, 0);
+      float mx[4];
+#pragma unroll
+      for (int ch = 0; ch < 4; ++ch) mx[ch] = max3(s[0][4 * ch], s[0][4 * ch + 1], s[0][4 * ch + 2]);
+#pragma unroll
+      for (int ch = 0; ch < 4; ++ch) mx[ch] = max3(mx[ch], s[0][4 * ch + 3], s[1][4 * ch]);
+#pragma unroll
+      for (int ch = 0; ch < 4; ++ch) mx[ch] = max3(mx[ch], s[1][4 * ch + 1], s[1][4 * ch + 2]);
+      const float m_new = lane32_max(max3(max3(mx[0], s[1][3], s[1][7]), max3(mx[1], s[1][11], s[1][15]), max3(mx[2], mx[3], m_run)));
+      bool changed = false;
+      float alpha = 1.f;
+      const float mc = m_new * c;
+      if constexpr (kFirst) {
+        m_run = m_new;  // O and l are still zero
+      } else {
+        changed = __any(m_new != m_run);
+        if (changed) {
+          alpha = __builtin_amdgcn_exp2f((m_run - m_new) * c);
+          l_run *= alpha;
+          m_run = m_new;
+        }
+      }
+      float sum0, sum1;
+      v8i p8_cur;
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        if (u == 1) issue_k(min(j + 3, n_tiles), k_dst, j + 3 < n_tiles);
+        if (u == 2) issue_v(min(j + 1, n_tiles), v_dst, j + 1 < n_tiles);
+        // LDS operands of the matrix instructions in front of the next chunk
+        if constexpr (!kFirst) {
+#pragma unroll
+          for (int mt = 1; mt < kMTiles; ++mt)
+            if (mt * kPvEvery - 1 == u) vfrag[mt] = load_vf(vb_prev, mt);
+        }
+#pragma unroll
+        for (int ks = 0; ks < kKSteps; ++ks)
+          if (4 + ks * kSEvery - 1 == u) kfrag[0][ks] = load_kf(kb_next, 0, ks);
+        if (u >= 8 - kKSteps) kfrag[1][u - (8 - kKSteps)] = load_kf(kb_next, 1, u - (8 - kKSteps));
+        // one matrix instruction in front of the chunk
+        if (u < 4 && u % kPvEvery == 0) {
+          if constexpr (!kFirst) o_acc[u / kPvEvery] = mfma_fp8<E5M2>(vfrag[u / kPvEvery], p8, o_acc[u / kPvEvery]);
+        }
+        if (u >= 4 && (u - 4) % kSEvery == 0 && (u - 4) / kSEvery < kKSteps) {
+          // (after the last block this is the product of a stale tile: never used)
+          const int ks = (u - 4) / kSEvery;
+          if (ks == 0) {
+            v16f z;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) z[i] = 0.f;
+            s[0] = mfma_fp8<E5M2>(kfrag[0][ks], qf[ks], z);
+          } else {
+            s[0] = mfma_fp8<E5M2>(kfrag[0][ks], qf[ks], s[0]);
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // chunk u of the softmax: weights 4w .. 4w+3 of sub-tile t
+        const int t = u >> 2, w = u & 3;
+        float x[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) x[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][4 * w + i], c, -mc));
+        sum0 = (u == 0) ? x[0] : sum0 + x[0];
+        sum1 = (u == 0) ? x[1] : sum1 + x[1];
+        sum0 += x[2];
+        sum1 += x[3];
+        int packed = pack4_fp8<E5M2>(x[0], x[1], x[2], x[3]);
+        // the weights are only read in the next iteration; without this pin the compiler sinks the conversions there
+        asm volatile("" : "+v"(packed));
+        p8_cur[u] = packed;
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+      for (int ks = 0; ks < kKSteps; ++ks) {
+        if (ks == 0) {
+          v16f z;
+#pragma unroll
+          for (int i = 0; i < 16; ++i) z[i] = 0.f;
+          s[1] = mfma_fp8<E5M2>(kfrag[1][ks], qf[ks], z);
+        } else {
+          s[1] = mfma_fp8<E5M2>(kfrag[1][ks], qf[ks], s[1]);
+        }
+      }
+      l_run += sum0 + sum1;
+      asm volatile("" : "+v"(l_run));  // keeps the additions above where they are written
+      // O now holds the PV product of block j-1: bring it to the new row max
+      if (changed) {
+#pragma unroll
+        for (int mt = 0; mt < kMTiles; ++mt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) o_acc[mt][i] *= alpha;
+      }
+      p8 = p8_cur;
+    };
+    // Waits until at most `tiles` tile copies (kPasses loads each) are in flight, then the barrier: it publishes the landed
+    // tiles and frees the stages read before it.  vmcnt counts this lane's loads in issue order.
+    auto wait_in_flight = [&](auto tiles_c) __attribute__((always_inline)) {
+      constexpr int n = decltype(tiles_c)::value * kPasses;
+      static_assert(n < 16, "vmcnt immediate");
+      __builtin_amdgcn_s_waitcnt(0x0F70 | n);
+      __builtin_amdgcn_s_barrier();
+    };
+    using T = std::true_type;
+    using F = std::false_type;
+    issue_k(0, k_lds0, true);
+    issue_k(min(1, n_tiles), k_lds1, 1 < n_tiles);
+    issue_k(min(2, n_tiles), k_lds2, 2 < n_tiles);
+    issue_v(0, v_lds0, true);
+    wait_in_flight(std::integral_constant<int, 2>());  // K(0) and K(1) landed
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s[t][i] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < kKSteps; ++ks) s[t] = mfma_fp8<E5M2>(load_kf(k_lds0, t, ks), qf[ks], s[t]);
+    }
+    __builtin_amdgcn_s_barrier();  // every wavefront has read K(0): step 0 may overwrite its stage
+    // One step with compile-time LDS stages (PH = j % 3).
+    auto step = [&](auto first_c, auto ph_c, int j) __attribute__((always_inline)) {
+      constexpr int PH = decltype(ph_c)::value;
+      uint8_t* const kst[3] = {k_lds0, k_lds1, k_lds2};
+      uint8_t* const vst[3] = {v_lds0, v_lds1, v_lds2};
+      iteration(first_c, j, kst[(PH + 1) % 3], vst[(PH + 2) % 3], kst[PH], vst[(PH + 1) % 3]);
+      wait_in_flight(std::integral_constant<int, 2>());  // the two copies of this step may stay in flight
+    };
+    constexpr std::integral_constant<int, 0> ph0{};
+    constexpr std::integral_constant<int, 1> ph1{};
+    constexpr std::integral_constant<int, 2> ph2{};
+    step(T(), ph0, 0);
+    int j = 1;
+    for (; j + 2 < n_tiles; j += 3) {
+      step(F(), ph1, j);
+      step(F(), ph2, j + 1);
+      step(F(), ph0, j + 2);
+    }
+    if (j < n_tiles) {
+      step(F(), ph1, j);
+      if (j + 1 < n_tiles) step(F(), ph2, j + 1);
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // the last copies (of nothing) must not outlive the workgroup's LDS
+    // the PV product of the last block
+    {
+      const int st = (n_tiles - 1) % 3;
+      const uint8_t* vb = st == 0 ? v_lds0 : (st == 1 ? v_lds1 : v_lds2);
+#pragma unroll
+      for (int mt = 0; mt < kMTiles; ++mt) o_acc[mt] = mfma_fp8<E5M2>(load_vf(vb, mt), p8, o_acc[mt]);
+    }
+  } else if constexpr (PIPE) {
     // ---- software-pipelined loop ----
     // Iteration j is the softmax of block j in 8 chunks of 4 weights with a matrix instruction in front of the chunks: first
     // the PV products of block j-1, then the S^T products of block j+1 (head dim 128: one per chunk, 64: every second
@@ -501,7 +680,6 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PIPE ?
     // starts the copies of K(j+4) and V(j+2) (their stages held K(j) and V(j-2), last read in iteration j-1), reads K(j+1)
     // and V(j-1), and ends when K(j+2) and V(j) have landed.  Every block takes this path, masked blocks included (their
     // weights become exact zeros), so the loop needs no second form.
-    static_assert(!PIPE || D == 64 || D == 128, "the pipelined loop is built for head dims 64 and 128");
     constexpr int kSlots = kMTiles + 2 * kKSteps;  // matrix instructions per iteration
     constexpr int kChunksPerSlot = 8 / kSlots;     // 1 (head dim 128) or 2 (64)
     v16f sbuf[2][2];
@@ -604,8 +782,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PIPE ?
           for (int i = 0; i < 16; ++i) o_acc[mt][i] *= alpha;
       }
     };
-    // Every step starts two tile copies, also past the last block (those read beyond the buffer: zeros, no memory traffic,
-    // never used), so the number of loads in flight is the same at every step.  vmcnt counts this lane's loads in issue order.
+    // Every step starts two tile copies, also past the last block this workgroup walks (those copy nothing, see issue_k), so the
+    // number of loads in flight is the same at every step.  vmcnt counts this lane's loads in issue order.
     // Waits until at most `tiles` tile copies (kPasses loads each) are in flight, then the barrier: it publishes the landed
     // tiles and frees the stages read before it.
     auto wait_in_flight = [&](auto tiles_c) __attribute__((always_inline)) {
@@ -625,12 +803,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PIPE ?
     using T = std::true_type;
     using F = std::false_type;
     // the copies of steps -4 .. -1
-    issue_k(0, k_lds0);
-    issue_k(min(1, n_tiles), k_lds1);
-    issue_k(min(2, n_tiles), k_lds2);
-    issue_v(0, v_lds0);
-    issue_k(min(3, n_tiles), k_lds3);
-    issue_v(min(1, n_tiles), v_lds1);
+    issue_k(0, k_lds0, true);
+    issue_k(min(1, n_tiles), k_lds1, 1 < n_tiles);
+    issue_k(min(2, n_tiles), k_lds2, 2 < n_tiles);
+    issue_v(0, v_lds0, true);
+    issue_k(min(3, n_tiles), k_lds3, 3 < n_tiles);
+    issue_v(min(1, n_tiles), v_lds1, 1 < n_tiles);
     wait_in_flight(std::integral_constant<int, 5>());  // K(0) landed
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
@@ -646,8 +824,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PIPE ?
       constexpr bool kFirst = decltype(first_c)::value;
       uint8_t* const kst[4] = {k_lds0, k_lds1, k_lds2, k_lds3};
       uint8_t* const vst[4] = {v_lds0, v_lds1, v_lds2, v_lds3};
-      issue_k(min(j + 4, n_tiles), kst[PH]);  // (block n_tiles lies wholly beyond the buffer)
-      issue_v(min(j + 2, n_tiles), vst[(PH + 2) % 4]);
+      issue_k(min(j + 4, n_tiles), kst[PH], j + 4 < n_tiles);
+      issue_v(min(j + 2, n_tiles), vst[(PH + 2) % 4], j + 2 < n_tiles);
       iteration(first_c, j, kst[(PH + 1) % 4], vst[(PH + 3) % 4], sbuf[PH % 2], sbuf[(PH + 1) % 2], p8buf[(PH + 1) % 2],
                 p8buf[PH % 2]);
       end_step();
@@ -801,33 +979,38 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PIPE ?
 }
 
 template <int D, bool CAUSAL, bool E5M2, int OUT>
-int launch(const KernelArgs& a, bool v_transposed, bool pipelined, hipStream_t stream) {
+int launch(const KernelArgs& a, bool v_transposed, int loop, hipStream_t stream) {
   const dim3 grid((unsigned)(a.bh_total * a.n_qblocks));
   // hipLaunchKernel returns the status of this launch itself; the thread's sticky "last error" (which an earlier,
   // unrelated call may have left behind) is neither read nor cleared.
   KernelArgs args = a;
   void* argv[] = {&args};
-  const void* fn = v_transposed ? (const void*)&fa8_fwd_kernel<D, CAUSAL, E5M2, OUT, true, false>
-                                : (const void*)&fa8_fwd_kernel<D, CAUSAL, E5M2, OUT, false, false>;
+  const void* fn = v_transposed ? (const void*)&fa8_fwd_kernel<D, CAUSAL, E5M2, OUT, true, kLoopRolling>
+                                : (const void*)&fa8_fwd_kernel<D, CAUSAL, E5M2, OUT, false, kLoopRolling>;
   if constexpr (D == 64 || D == 128) {
-    if (pipelined)
-      fn = v_transposed ? (const void*)&fa8_fwd_kernel<D, CAUSAL, E5M2, OUT, true, true>
-                        : (const void*)&fa8_fwd_kernel<D, CAUSAL, E5M2, OUT, false, true>;
+    if (loop == FA8_SCHEDULE_PIPELINED)
+      fn = v_transposed ? (const void*)&fa8_fwd_kernel<D, CAUSAL, E5M2, OUT, true, kLoopPipelined>
+                        : (const void*)&fa8_fwd_kernel<D, CAUSAL, E5M2, OUT, false, kLoopPipelined>;
+    if constexpr (!CAUSAL) {
+      if (loop == FA8_SCHEDULE_DENSE)
+        fn = v_transposed ? (const void*)&fa8_fwd_kernel<D, false, E5M2, OUT, true, kLoopDense>
+                          : (const void*)&fa8_fwd_kernel<D, false, E5M2, OUT, false, kLoopDense>;
+    }
   }
   return (int)hipLaunchKernel(fn, grid, dim3(kThreads), argv, 0, stream);
 }
 
 template <int D, bool CAUSAL>
-int launch_types(const Fa8FwdParams* p, const KernelArgs& a, bool pipelined, hipStream_t stream) {
+int launch_types(const Fa8FwdParams* p, const KernelArgs& a, int loop, hipStream_t stream) {
   const bool e5m2 = p->in_dtype == FA8_DTYPE_E5M2, vt = p->v_layout == FA8_V_TRANSPOSED;
   if (p->out_dtype == FA8_OUT_FP16)
-    return e5m2 ? launch<D, CAUSAL, true, FA8_OUT_FP16>(a, vt, pipelined, stream)
-                : launch<D, CAUSAL, false, FA8_OUT_FP16>(a, vt, pipelined, stream);
+    return e5m2 ? launch<D, CAUSAL, true, FA8_OUT_FP16>(a, vt, loop, stream)
+                : launch<D, CAUSAL, false, FA8_OUT_FP16>(a, vt, loop, stream);
   // fp8 output: the reference stores O in the input element type (csrc/flash_attention.cu:557, :655-656); the two
   // mixed combinations are not built
   if (e5m2)
-    return p->out_dtype == FA8_OUT_E5M2 ? launch<D, CAUSAL, true, FA8_OUT_E5M2>(a, vt, pipelined, stream) : FA8_ERR_UNSUPPORTED;
-  return p->out_dtype == FA8_OUT_E4M3 ? launch<D, CAUSAL, false, FA8_OUT_E4M3>(a, vt, pipelined, stream) : FA8_ERR_UNSUPPORTED;
+    return p->out_dtype == FA8_OUT_E5M2 ? launch<D, CAUSAL, true, FA8_OUT_E5M2>(a, vt, loop, stream) : FA8_ERR_UNSUPPORTED;
+  return p->out_dtype == FA8_OUT_E4M3 ? launch<D, CAUSAL, false, FA8_OUT_E4M3>(a, vt, loop, stream) : FA8_ERR_UNSUPPORTED;
 }
 
 // KV blocks walked by all workgroups of a launch together.
@@ -847,34 +1030,42 @@ long long launch_kv_blocks(const Fa8FwdParams* p) {
   return bh * (n1 + cnt * base + (n1 + first - 1) * cnt + (nq - first) * tk);
 }
 
-// Compute units of the current device (0 if the runtime cannot tell), asked once per device.
+// Compute units of the current device (0 if the runtime cannot tell), asked once per device.  The current device must be the
+// one that owns the stream and the tensors of the call (the PyTorch binding and the ctypes mirror see to it).
 int compute_units() {
-  static int cached[64];
+  static std::atomic<int> cached[64];  // zero-initialised; racing first calls store the same value
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
-  if (cached[dev] == 0) {
-    int n = 0;
+  int n = cached[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
     if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1) return 0;
-    cached[dev] = n;
+    cached[dev].store(n, std::memory_order_relaxed);
   }
-  return cached[dev];
+  return n;
 }
 
-// Which main loop a valid call runs (see fa8_fwd_kernel).  The pipelined one for launches that cannot keep three wavefronts on
-// every SIMD for most of their run: at most four workgroups per compute unit (two resident at a time), or little work per
-// compute unit (then filling and draining the chip, and for causal launches the thinning out of the workgroups, is a large
-// share of the run).  Measured 5 - 15 % faster there; the rolling loop is equal or up to 5 % faster elsewhere.  The pipelined
-// loop exists for head dims 64 and 128 and relies on exp2(-inf * scale) = 0 for masked logits, i.e. on a positive softmax
-// scale; elsewhere the hint is ignored.
-bool runs_pipelined(const Fa8FwdParams* p) {
-  if ((p->head_dim != 64 && p->head_dim != 128) || !(p->softmax_scale > 0.f)) return false;
-  if (p->schedule != FA8_SCHEDULE_AUTO) return p->schedule == FA8_SCHEDULE_PIPELINED;
+// Which main loop a valid call runs (see fa8_fwd_kernel): FA8_SCHEDULE_ROLLING, _PIPELINED or _DENSE.
+// The pipelined loops exist for head dims 64 and 128 and for a positive softmax scale (the pipelined loop relies on
+// exp2(-inf * scale) = 0 for masked logits); elsewhere every hint is ignored and the rolling loop runs.
+// Dense: full (non-causal) attention over a whole number of KV blocks, where no logit is ever masked; measured 1 - 2 % faster
+// than the rolling loop on launches that fill the chip and 3 - 5 % faster than the pipelined loop on small ones, so it is
+// the choice wherever it applies.  A hint for it that does not apply falls back to the automatic choice.
+// Pipelined: launches that cannot keep three wavefronts on every SIMD for most of their run: at most four workgroups per
+// compute unit (two resident at a time), or little work per compute unit (then filling and draining the chip, and for
+// causal launches the thinning out of the workgroups, is a large share of the run).  Measured 5 - 15 % faster than the
+// rolling loop there; the rolling loop is equal or up to 5 % faster elsewhere.
+int choose_loop(const Fa8FwdParams* p) {
+  if ((p->head_dim != 64 && p->head_dim != 128) || !(p->softmax_scale > 0.f)) return FA8_SCHEDULE_ROLLING;
+  const bool dense_ok = !p->is_causal && p->seqlen_k % kKvBlock == 0;
+  if (p->schedule == FA8_SCHEDULE_ROLLING || p->schedule == FA8_SCHEDULE_PIPELINED) return p->schedule;
+  if (dense_ok) return FA8_SCHEDULE_DENSE;
   const long long cus = compute_units();
   const long long wgs = (long long)p->batch * p->heads * ((p->seqlen_q + kQBlock - 1) / kQBlock);
   // KV blocks per compute unit below which the pipelined loop was measured to win (head dim 64 has half the matrix work
   // per block)
   const long long few_blocks = p->head_dim == 64 ? 264 : 144;
-  return cus > 0 && (wgs <= 4 * cus || (wgs <= few_blocks * cus && launch_kv_blocks(p) <= few_blocks * cus));
+  const bool small = cus > 0 && (wgs <= 4 * cus || (wgs <= few_blocks * cus && launch_kv_blocks(p) <= few_blocks * cus));
+  return small ? FA8_SCHEDULE_PIPELINED : FA8_SCHEDULE_ROLLING;
 }
 
 bool span_ok(long long outer_stride, long long inner_extent) { return outer_stride >= inner_extent; }
@@ -887,8 +1078,8 @@ extern "C" int fa8_fwd_validate(const Fa8FwdParams* p) {
   if (p->is_causal != 0 && p->is_causal != 1) return FA8_ERR_SHAPE;
   if (p->heads_k < 0 || (p->heads_k > 0 && p->heads % p->heads_k != 0)) return FA8_ERR_SHAPE;
   if (p->causal_align != FA8_CAUSAL_TOP_LEFT && p->causal_align != FA8_CAUSAL_BOTTOM_RIGHT) return FA8_ERR_DTYPE;
-  if (p->schedule != FA8_SCHEDULE_AUTO && p->schedule != FA8_SCHEDULE_ROLLING && p->schedule != FA8_SCHEDULE_PIPELINED)
-    return FA8_ERR_DTYPE;
+  if (p->schedule < FA8_SCHEDULE_AUTO || p->schedule > FA8_SCHEDULE_DENSE) return FA8_ERR_DTYPE;
+  if (p->reserved0 != 0) return FA8_ERR_UNSUPPORTED;  // a field of a later version of the parameter block
   if ((long long)p->batch * p->heads > 0x7fffffffLL / ((p->seqlen_q + kQBlock - 1) / kQBlock)) return FA8_ERR_SHAPE;
   if (p->in_dtype != FA8_DTYPE_E4M3 && p->in_dtype != FA8_DTYPE_E5M2) return FA8_ERR_DTYPE;
   if (p->out_dtype != FA8_OUT_FP16 && p->out_dtype != FA8_OUT_E4M3 && p->out_dtype != FA8_OUT_E5M2) return FA8_ERR_DTYPE;
@@ -959,10 +1150,10 @@ extern "C" int fa8_fwd(const Fa8FwdParams* p, void* hip_stream) {
   a.v_bs = p->v_batch_stride; a.v_hs = p->v_head_stride; a.v_rs = p->v_row_stride;
   a.o_bs = p->o_batch_stride; a.o_hs = p->o_head_stride; a.o_rs = p->o_row_stride;
   hipStream_t stream = (hipStream_t)hip_stream;
-  const bool pipelined = runs_pipelined(p);
+  const int loop = choose_loop(p);
   switch (p->head_dim) {
 #define FA8_HEAD_DIM_CASE(D_) \
-  case D_: return p->is_causal ? launch_types<D_, true>(p, a, pipelined, stream) : launch_types<D_, false>(p, a, pipelined, stream)
+  case D_: return p->is_causal ? launch_types<D_, true>(p, a, loop, stream) : launch_types<D_, false>(p, a, loop, stream)
     FA8_HEAD_DIM_CASE(32);  // the head-dim buckets of the reference (csrc/static_switch.h:50-77)
     FA8_HEAD_DIM_CASE(64);
     FA8_HEAD_DIM_CASE(96);
@@ -979,7 +1170,7 @@ extern "C" int fa8_fwd(const Fa8FwdParams* p, void* hip_stream) {
 extern "C" int fa8_fwd_schedule(const Fa8FwdParams* p) {
   const int rc = fa8_fwd_validate(p);
   if (rc != FA8_OK) return rc;
-  return runs_pipelined(p) ? FA8_SCHEDULE_PIPELINED : FA8_SCHEDULE_ROLLING;
+  return choose_loop(p);
 }
 
 extern "C" int fa8_query(int what) {

@@ -39,13 +39,16 @@ extern "C" {
 #define FA8_CAUSAL_BOTTOM_RIGHT 1 /* key j <= i + seqlen_k - seqlen_q: the last query sees every key (decode, chunked prefill) */
 
 /* which main loop the kernel runs: a performance hint, the results are bitwise the same
- *   AUTO      the library chooses from the size of the launch
- *   ROLLING   one KV block after the other, three wavefronts per SIMD: for launches that fill the chip
- *   PIPELINED software-pipelined over neighbouring KV blocks, two wavefronts per SIMD: for small launches
- *             (built for head dims 64 and 128; ignored for the others) */
+ *   AUTO      the library chooses from the shape of the launch
+ *   ROLLING   one KV block after the other, three wavefronts per SIMD: for masked launches that fill the chip
+ *   PIPELINED software-pipelined over neighbouring KV blocks, two wavefronts per SIMD: for small masked launches
+ *   DENSE     the same pipeline in three wavefronts per SIMD, for launches without any masked logit: full (non-causal)
+ *             attention with seqlen_k a multiple of 64; asked for elsewhere, the library chooses as for AUTO
+ *   (PIPELINED and DENSE are built for head dims 64 and 128 and a positive softmax scale; ignored elsewhere) */
 #define FA8_SCHEDULE_AUTO 0
 #define FA8_SCHEDULE_ROLLING 1
 #define FA8_SCHEDULE_PIPELINED 2
+#define FA8_SCHEDULE_DENSE 3
 
 /* error codes (all negative) */
 #define FA8_OK 0
@@ -98,7 +101,7 @@ typedef struct Fa8FwdParams {
   int32_t causal_align; /* FA8_CAUSAL_* */
   /* ---- library version 3; all-zero = the library chooses ---- */
   int32_t schedule;  /* FA8_SCHEDULE_*: a performance hint, never changes the result */
-  int32_t reserved0; /* must be 0 */
+  int32_t reserved0; /* must be 0 (anything else: FA8_ERR_UNSUPPORTED) */
 } Fa8FwdParams;
 
 /*
@@ -117,8 +120,8 @@ int fa8_fwd_validate(const Fa8FwdParams* p);
 int fa8_fwd(const Fa8FwdParams* p, void* hip_stream);
 
 /*
- * Which main loop fa8_fwd would run for these arguments on the current device: FA8_SCHEDULE_ROLLING or
- * FA8_SCHEDULE_PIPELINED (both > 0), or the FA8_ERR_* code fa8_fwd_validate gives.  Launches nothing.  No counterpart in
+ * Which main loop fa8_fwd would run for these arguments on the current device: FA8_SCHEDULE_ROLLING,
+ * FA8_SCHEDULE_PIPELINED or FA8_SCHEDULE_DENSE (all > 0), or the FA8_ERR_* code fa8_fwd_validate gives.  Launches nothing.  No counterpart in
  * the reference (one kernel, one loop: csrc/flash_attention.cu:468-534); it makes the library's choice visible to
  * benchmarks and tests.
  */

@@ -144,7 +144,7 @@ def test_compiled_binding_mirrors_reference_errors():
 
 
 def test_schedule_query_follows_explicit_hints_without_a_gpu():
-    """fa8_fwd_schedule: an explicit hint is answered without touching the GPU; it holds only where the pipelined loop exists."""
+    """fa8_fwd_schedule: an explicit hint is answered without touching the GPU; it holds only where the loop it names exists."""
     sched = fa.lib().fa8_fwd_schedule
     for d, scale, hint, want in ((128, 0.1, fa.FA8_SCHEDULE_PIPELINED, fa.FA8_SCHEDULE_PIPELINED),
                                  (64, 0.1, fa.FA8_SCHEDULE_PIPELINED, fa.FA8_SCHEDULE_PIPELINED),
@@ -156,7 +156,20 @@ def test_schedule_query_follows_explicit_hints_without_a_gpu():
         q, k, v, o = cpu_tensors(d=d)
         p = fa.make_params(q, k, v, o, True, scale, schedule=hint)
         assert sched(ctypes.byref(p)) == want, (d, scale, hint)
+    # the dense loop: full attention, seqlen_k a multiple of the KV block, head dim 64 / 128, positive scale; chosen without a hint
+    for d, n, scale, hint, want in ((128, 128, 0.1, fa.FA8_SCHEDULE_AUTO, fa.FA8_SCHEDULE_DENSE),
+                                    (64, 64, 0.1, fa.FA8_SCHEDULE_DENSE, fa.FA8_SCHEDULE_DENSE),
+                                    (128, 128, 0.1, fa.FA8_SCHEDULE_ROLLING, fa.FA8_SCHEDULE_ROLLING),
+                                    (128, 128, 0.1, fa.FA8_SCHEDULE_PIPELINED, fa.FA8_SCHEDULE_PIPELINED),
+                                    (96, 128, 0.1, fa.FA8_SCHEDULE_DENSE, fa.FA8_SCHEDULE_ROLLING),
+                                    (128, 128, 0.0, fa.FA8_SCHEDULE_DENSE, fa.FA8_SCHEDULE_ROLLING)):
+        q, k, v, o = cpu_tensors(n=n, d=d)
+        p = fa.make_params(q, k, v, o, False, scale, schedule=hint)
+        assert sched(ctypes.byref(p)) == want, (d, n, scale, hint)
     q, k, v, o = cpu_tensors()
     p = fa.make_params(q, k, v, o, False, 0.1, schedule=9)
     assert sched(ctypes.byref(p)) == -6 and validate(p) == -6  # FA8_ERR_DTYPE: unknown schedule code
     assert sched(None) == -1
+    p = fa.make_params(q, k, v, o, False, 0.1)
+    p.reserved0 = 1
+    assert validate(p) == -7  # FA8_ERR_UNSUPPORTED: a field of a later version of the parameter block is set

@@ -217,22 +217,23 @@ def test_error_paths_raise_and_launch_nothing():
     assert np.abs(o.float().cpu().numpy() - ref).mean() <= 2e-3
 
 
-@pytest.mark.parametrize("schedule", [fa.FA8_SCHEDULE_ROLLING, fa.FA8_SCHEDULE_PIPELINED], ids=["rolling", "pipelined"])
-def test_capturable_in_a_hip_graph(schedule):
+@pytest.mark.parametrize("schedule,causal", [(fa.FA8_SCHEDULE_ROLLING, True), (fa.FA8_SCHEDULE_PIPELINED, True),
+                                             (fa.FA8_SCHEDULE_DENSE, False)], ids=["rolling", "pipelined", "dense"])
+def test_capturable_in_a_hip_graph(schedule, causal):
     """The launcher allocates nothing and never synchronises, so the operator can be recorded into a HIP graph
-    (here through torch.cuda.graph, whose allocator provides the output inside the capture) and replayed; both main loops."""
+    (here through torch.cuda.graph, whose allocator provides the output inside the capture) and replayed; all main loops."""
     ext = fa.load_extension()
     q, k, v = (rand_fp8((2, 4, 384, 128), s).to(DEV) for s in (50, 51, 52))
-    eager = ext.flash_attention_v2_cutlass(q, k, v, True, 0.09, schedule=schedule)[0].clone()
+    eager = ext.flash_attention_v2_cutlass(q, k, v, causal, 0.09, schedule=schedule)[0].clone()
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):  # warm-up outside the capture, as torch asks
-        ext.flash_attention_v2_cutlass(q, k, v, True, 0.09, schedule=schedule)
+        ext.flash_attention_v2_cutlass(q, k, v, causal, 0.09, schedule=schedule)
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
-        out = ext.flash_attention_v2_cutlass(q, k, v, True, 0.09, schedule=schedule)[0]
+        out = ext.flash_attention_v2_cutlass(q, k, v, causal, 0.09, schedule=schedule)[0]
     for i in range(3):
         out.fill_(float("nan"))
         torch.cuda.synchronize()
@@ -241,4 +242,4 @@ def test_capturable_in_a_hip_graph(schedule):
         assert torch.equal(out, eager), f"replay {i}"
         # eager work and new inputs between replays: the graph reads q/k/v in place
         q.copy_(rand_fp8((2, 4, 384, 128), 60 + i).to(DEV))
-        eager = ext.flash_attention_v2_cutlass(q, k, v, True, 0.09, schedule=schedule)[0].clone()
+        eager = ext.flash_attention_v2_cutlass(q, k, v, causal, 0.09, schedule=schedule)[0].clone()

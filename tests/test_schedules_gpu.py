@@ -1,7 +1,9 @@
-"""The two main loops of the kernel (FA8_SCHEDULE_ROLLING / FA8_SCHEDULE_PIPELINED, include/fa8_api.h) perform the same
+"""The three main loops of the kernel (FA8_SCHEDULE_ROLLING / _PIPELINED / _DENSE, include/fa8_api.h) perform the same
 arithmetic in the same order: their outputs must be bitwise equal, for every feature of the operator.  The parity of the
-result itself is the business of the parity tests; they reach the pipelined loop through the library's own choice (small
-launches) and the rolling loop through the large configurations."""
+result itself is the business of the parity tests; they reach the dense loop through the library's own choice (full
+attention over whole KV blocks), the pipelined loop through small masked launches and the rolling loop through the large
+causal configurations.  A dense hint that does not apply (causal, ragged seqlen_k) is answered with the automatic choice,
+so asking for it is always valid."""
 import numpy as np
 import pytest
 import torch
@@ -23,6 +25,10 @@ def _inputs(seed, B, H, Hk, Nq, Nk, d, dtype, heavy=False):
 CASES = [
     # B, H, Hk, Nq, Nk, d, causal, bottom_right, vt, in dtype, out dtype
     (1, 2, 2, 64, 64, 128, False, False, False, torch.float8_e4m3fn, torch.float16),     # a single block
+    (1, 2, 2, 1, 64, 64, False, False, False, torch.float8_e4m3fn, torch.float16),       # one query, one block
+    (1, 2, 2, 77, 128, 128, False, False, False, torch.float8_e4m3fn, torch.float16),    # 2 blocks, ragged queries
+    (1, 2, 1, 200, 256, 64, False, False, True, torch.float8_e4m3fn, torch.float8_e4m3fn),  # 4 blocks, v^T, fp8 out, grouped
+    (1, 2, 2, 300, 448, 128, False, False, True, torch.float8_e5m2, torch.float8_e5m2),  # 7 blocks
     (1, 2, 2, 65, 65, 128, True, False, False, torch.float8_e4m3fn, torch.float16),      # one row into the second block
     (2, 3, 3, 128, 128, 64, True, False, False, torch.float8_e4m3fn, torch.float16),
     (1, 2, 2, 192, 192, 128, False, False, False, torch.float8_e4m3fn, torch.float16),   # 3 blocks
@@ -47,28 +53,30 @@ CASES = [
 
 
 @pytest.mark.parametrize("case", CASES, ids=lambda c: f"B{c[0]}H{c[1]}k{c[2]}Nq{c[3]}Nk{c[4]}d{c[5]}{'c' if c[6] else 'f'}{'br' if c[7] else ''}{'vt' if c[8] else ''}")
-def test_rolling_and_pipelined_loops_agree_bitwise(case):
+def test_the_loops_agree_bitwise(case):
     B, H, Hk, Nq, Nk, d, causal, br, vt, in_dt, out_dt = case
     if vt and Nk % 16:
         pytest.skip("transposed v needs seqlen_k % 16 == 0")
     q, k, v = _inputs(hash(case[:7]) % 1000, B, H, Hk, Nq, Nk, d, in_dt, heavy=(Nq % 2 == 1))
     v_arg = v.transpose(2, 3).contiguous() if vt else v
     outs = {}
-    for name, sched in (("rolling", fa.FA8_SCHEDULE_ROLLING), ("pipelined", fa.FA8_SCHEDULE_PIPELINED)):
+    for name, sched in (("rolling", fa.FA8_SCHEDULE_ROLLING), ("pipelined", fa.FA8_SCHEDULE_PIPELINED), ("dense", fa.FA8_SCHEDULE_DENSE)):
         o, lse = fa.flash_attention_v2_cutlass(q.to(DEV), k.to(DEV), v_arg.to(DEV), causal, d ** -0.5, v_transposed=vt,
                                                out_dtype=out_dt, return_lse=True, causal_bottom_right=br, schedule=sched)
         torch.cuda.synchronize()
         outs[name] = (o.cpu().view(torch.uint8 if out_dt != torch.float16 else torch.int16).numpy(), lse.cpu().numpy())
     o_r, lse_r = outs["rolling"]
-    o_p, lse_p = outs["pipelined"]
-    assert np.array_equal(o_r, o_p), f"{int((o_r != o_p).sum())} output elements differ between the two loops"
-    assert np.array_equal(lse_r.view(np.int32), lse_p.view(np.int32)), "log-sum-exp differs between the two loops"
+    for name in ("pipelined", "dense"):
+        o_p, lse_p = outs[name]
+        assert np.array_equal(o_r, o_p), f"{int((o_r != o_p).sum())} output elements differ between the rolling and the {name} loop"
+        assert np.array_equal(lse_r.view(np.int32), lse_p.view(np.int32)), f"log-sum-exp differs between the rolling and the {name} loop"
 
 
-@pytest.mark.parametrize("sched", [fa.FA8_SCHEDULE_ROLLING, fa.FA8_SCHEDULE_PIPELINED], ids=["rolling", "pipelined"])
+@pytest.mark.parametrize("sched", [fa.FA8_SCHEDULE_ROLLING, fa.FA8_SCHEDULE_PIPELINED, fa.FA8_SCHEDULE_DENSE],
+                         ids=["rolling", "pipelined", "dense"])
 @pytest.mark.parametrize("causal", [False, True], ids=["full", "causal"])
 def test_each_loop_against_the_oracle(sched, causal):
-    B, H, N, d = 1, 2, 333, 128
+    B, H, N, d = 1, 2, 320, 128  # 5 whole blocks: the dense hint holds for the full-attention case
     q, k, v = _inputs(7, B, H, H, N, N, d, torch.float8_e4m3fn)
     scale = 0.11
     o = fa.flash_attention_v2_cutlass(q.to(DEV), k.to(DEV), v.to(DEV), causal, scale, schedule=sched)[0]
@@ -91,7 +99,8 @@ def test_non_positive_scale_and_other_head_dims_ignore_the_hint():
 
 
 def test_library_choice_by_launch_size():
-    """fa8_fwd_schedule on the GPU box: small launches take the pipelined loop, launches that fill the chip the rolling one."""
+    """fa8_fwd_schedule on the GPU box: full attention over whole KV blocks takes the dense loop; of the others, small launches
+    take the pipelined loop and launches that fill the chip the rolling one."""
     import ctypes
 
     def plan(B, H, N, d, causal):
@@ -100,8 +109,10 @@ def test_library_choice_by_launch_size():
         return fa.lib().fa8_fwd_schedule(ctypes.byref(fa.make_params(q, q, q, o, causal, d ** -0.5)))
 
     assert plan(1, 16, 1024, 128, True) == fa.FA8_SCHEDULE_PIPELINED      # 128 workgroups
-    assert plan(4, 16, 1024, 64, False) == fa.FA8_SCHEDULE_PIPELINED      # 512 workgroups (cfg2)
+    assert plan(4, 16, 1024, 64, False) == fa.FA8_SCHEDULE_DENSE          # cfg2
+    assert plan(4, 16, 1000, 64, False) == fa.FA8_SCHEDULE_PIPELINED      # 512 workgroups with a ragged last block
     assert plan(4, 32, 2048, 64, True) == fa.FA8_SCHEDULE_PIPELINED       # 2048 short causal workgroups: little work per CU
-    assert plan(2, 32, 4096, 128, False) == fa.FA8_SCHEDULE_ROLLING       # the headline shape
+    assert plan(2, 32, 4096, 128, False) == fa.FA8_SCHEDULE_DENSE         # the headline shape
+    assert plan(2, 32, 4097, 128, False) == fa.FA8_SCHEDULE_ROLLING       # ... with a ragged last block
     assert plan(1, 32, 8192, 128, True) == fa.FA8_SCHEDULE_ROLLING        # cfg4
     assert plan(1, 16, 1024, 96, True) == fa.FA8_SCHEDULE_ROLLING         # no pipelined loop for this head dim
