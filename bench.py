@@ -124,6 +124,45 @@ def read_power_w():
     return now, first(base + "power1_cap")
 
 
+def time_other_workload(name, ext, fa, inputs, torch, launches=20, settle_seconds=0.15):
+    """Kernel time of one more BASELINE workload, measured like the headline: clock-settle launches, then one HIP-event pair
+    per launch on torch's current stream.  Returns the entry of config.other_workloads."""
+    cfg = inputs.CONFIGS[name]
+    scale, causal = inputs.softmax_scale(cfg), cfg["causal"]
+    q, k, v = (t.to("cuda:0") for t in inputs.make_qkv(cfg))
+
+    def step():
+        return ext.flash_attention_v2_cutlass(q, k, v, causal, scale)[0]
+    plan = fa.lib().fa8_fwd_schedule(ctypes.byref(fa.make_params(q, k, v, step(), causal, scale)))
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < settle_seconds:
+        for _ in range(20):
+            step()
+        torch.cuda.synchronize()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(launches)]
+    for e0, e1 in evs:
+        e0.record()
+        step()
+        e1.record()
+    torch.cuda.synchronize()
+    ms = sorted(e0.elapsed_time(e1) for e0, e1 in evs)
+    avg = sum(ms) / len(ms)
+    flops, alg = inputs.flops(cfg), inputs.algorithmic_bytes(cfg)
+    traffic = MEASURED_TRAFFIC_BYTES.get(name)
+    return {"workload": f"{name}: B={cfg['B']} H={cfg['H']} N={cfg['N']} d={cfg['d']} {'causal' if causal else 'non-causal'}",
+            "main_loop": MAIN_LOOPS.get(plan, f"error {plan}"),
+            "kernel_ms_avg": round(avg, 5), "kernel_ms_min": round(ms[0], 5),
+            "tflops": round(flops / (avg * 1e-3) / 1e12, 1),
+            "pct_fp8_mfma_peak": round(100.0 * flops / (avg * 1e-3) / 1e12 / FP8_MFMA_PEAK_TFLOPS, 2),
+            "algorithmic_hbm_gbps": round(alg / (avg * 1e-3) / 1e9, 1),
+            "pct_hbm_peak": round(100.0 * alg / (avg * 1e-3) / 1e9 / HBM_PEAK_GBPS, 2),
+            # HBM bytes per launch from the committed rocprofv3 --pmc runs over the algorithmic bytes (not measured in this run)
+            "traffic_ratio": round(traffic / alg, 2) if traffic else None}
+
+
+MAIN_LOOPS = {1: "rolling", 2: "pipelined", 3: "dense"}  # FA8_SCHEDULE_* (include/fa8_api.h)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -131,6 +170,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="cfg3", help="cfg1..cfg5 (cfg3 is the headline)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-workloads", action="store_true",
+                    help="skip the kernel times of the other BASELINE workloads (config.other_workloads; headline runs only)")
     ap.add_argument("--settle-seconds", type=float, default=0.25,
                     help="untimed launches for this long after the warm-up, so that the shader clock has settled")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the baseline sample")
@@ -139,9 +180,9 @@ def main():
                          "(reference test.py:95-100: B=1, causal, scale=1/sqrt(N), inputs clamped to +-0.1) and print "
                          "one JSON line holding the table next to the reference's published Ada numbers")
     ap.add_argument("--instruction-mix", action="store_true",
-                    help="run only the instruction-mix probe (cutlass_flash_atten_fp8_amd/csrc/softmax_mix_probe.hip): what a "
-                         "SIMD needs for the vector and matrix instructions of one KV block with no memory traffic at all; "
-                         "prints its JSON lines")
+                    help="run only the instruction-mix probe (bench_mix_probe.hip beside this file, built with hipcc on first "
+                         "use): what a SIMD needs for the vector and matrix instructions of one KV block, then with the LDS "
+                         "operand reads, the tile copies and the barrier of the loop added; prints its JSON lines")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a plain 256 MiB device-to-device copy (10 times): the known-size kernel that the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run are scaled by")
@@ -153,10 +194,11 @@ def main():
 
     if args.instruction_mix:
         import subprocess
-        from cutlass_flash_atten_fp8_amd import build as native_build
-        if not os.path.exists(native_build.MIX_PROBE):
-            native_build.build_mix_probe()
-        sys.exit(subprocess.run([native_build.MIX_PROBE]).returncode)
+        src, exe = os.path.join(ROOT, "bench_mix_probe.hip"), os.path.join(ROOT, "bench_mix_probe")
+        if not os.path.exists(exe) or os.path.getmtime(exe) < os.path.getmtime(src):
+            subprocess.run([os.path.join(os.environ.get("ROCM_PATH", "/opt/rocm"), "bin", "hipcc"), "--offload-arch=gfx950", "-O3",
+                            "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-o", exe, src], check=True)
+        sys.exit(subprocess.run([exe]).returncode)
     import torch
     import cutlass_flash_atten_fp8_amd as fa
     from cutlass_flash_atten_fp8_amd import inputs
@@ -186,9 +228,9 @@ def main():
     def step():
         return ext.flash_attention_v2_cutlass(q, k, v, causal, scale)[0]
 
-    # which of the kernel's two main loops the library runs for this launch (include/fa8_api.h, FA8_SCHEDULE_*)
+    # which of the kernel's main loops the library runs for this launch (include/fa8_api.h, FA8_SCHEDULE_*)
     plan = fa.lib().fa8_fwd_schedule(ctypes.byref(fa.make_params(q, k, v, step(), causal, scale)))
-    main_loop = {fa.FA8_SCHEDULE_ROLLING: "rolling", fa.FA8_SCHEDULE_PIPELINED: "pipelined", fa.FA8_SCHEDULE_DENSE: "dense"}.get(plan, f"error {plan}")
+    main_loop = MAIN_LOOPS.get(plan, f"error {plan}")
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -278,6 +320,11 @@ def main():
             "kernel_ms_median": round(kern_ms[len(kern_ms) // 2], 5),
         },
     }
+
+    if args.workload == "cfg3" and not args.no_other_workloads:
+        # the other BASELINE workloads in the same process: kernel time, TFLOP/s and algorithmic HBM rate (value, ms_per_step and
+        # roofline above stay the headline's)
+        out["config"]["other_workloads"] = [time_other_workload(w, ext, fa, inputs, torch) for w in ("cfg2", "cfg4", "cfg5")]
 
     if not args.no_cpu_baseline:
         # The reference's CPU-runnable path (naive attention, reference test.py:25-33) restated in oracle/ and timed

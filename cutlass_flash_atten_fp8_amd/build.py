@@ -2,7 +2,6 @@
 
   libfa8.so                      hipcc --offload-arch=gfx950: kernels + C ABI (include/fa8_api.h)
   attention_cutlass_fp8.*.so     g++ host-only PyTorch binding that calls libfa8.so
-  softmax_mix_probe              hipcc: measurement tool of `bench.py --instruction-mix`
   ../tests/cabi_host             g++: standalone C++ host of the C ABI (tests/test_cabi_host_gpu.py)
 
 Run as `python -m cutlass_flash_atten_fp8_amd.build` or through __graft_entry__.build().
@@ -74,22 +73,15 @@ def build_cabi_host(force=False):
     return CABI_HOST
 
 
-MIX_PROBE = os.path.join(PKG_DIR, "softmax_mix_probe")
-
-
-def build_mix_probe():
-    """softmax_mix_probe: the measurement tool behind `bench.py --instruction-mix` (csrc/softmax_mix_probe.hip)."""
-    _run([os.path.join(ROCM, "bin", "hipcc"), "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
-          "-packed-fp32-ops", "-o", MIX_PROBE, os.path.join(CSRC, "softmax_mix_probe.hip")])
-    return MIX_PROBE
-
-
 def build_all():
     build_libfa8()
     build_binding()
-    build_mix_probe()
+    # the C++ host of the C ABI is a test helper: failing to build it must not fail the product build
     if os.path.exists(CABI_HOST_SRC):
-        build_cabi_host(force=True)
+        try:
+            build_cabi_host(force=True)
+        except RuntimeError as e:
+            sys.stderr.write("warning: tests/cabi_host was not built (%s)\n" % e)
     return LIBFA8, EXT_PATH
 
 

@@ -18,7 +18,7 @@ sys.path.insert(0, ROOT)
 
 def native_build(force=False):
     from cutlass_flash_atten_fp8_amd import build as nb
-    src = [os.path.join(nb.CSRC, f) for f in os.listdir(nb.CSRC)] + [os.path.join(nb.INCLUDE, "fa8_api.h")]
+    src = [os.path.join(nb.CSRC, f) for f in ("fa8_fwd_gfx950.hip", "attention_api.cpp")] + [os.path.join(nb.INCLUDE, "fa8_api.h")]
     newest = max(os.path.getmtime(f) for f in src)
     if force or not os.path.exists(nb.LIBFA8) or os.path.getmtime(nb.LIBFA8) < newest:
         nb.build_libfa8()
@@ -51,11 +51,11 @@ class BuildPyWithNative(build_py):
 
 setup(
     name="cutlass_flash_atten_fp8_amd",
-    version="0.2.0",
+    version="0.3.0",
     description="FP8 flash-attention forward for AMD MI355X (gfx950) behind the attention_cutlass_fp8 operator",
     packages=["cutlass_flash_atten_fp8_amd"],
     py_modules=["attention_cutlass_fp8"],
-    package_data={"cutlass_flash_atten_fp8_amd": ["*.so", "csrc/*"]},
+    package_data={"cutlass_flash_atten_fp8_amd": ["*.so", "csrc/fa8_fwd_gfx950.hip", "csrc/attention_api.cpp"]},
     cmdclass={"build_ext": BuildNative, "build_py": BuildPyWithNative},
     python_requires=">=3.9",
 )

@@ -90,7 +90,7 @@ def test_cfg2_full():
 def test_large_configs_sampled(name):
     cfg = inputs.CONFIGS[name]
     q, k, v = inputs.make_qkv(cfg)
-    check(q, k, v, inputs.softmax_scale(cfg), cfg["causal"], rows=sample_rows(cfg["N"], 512), label=name)
+    check(q, k, v, inputs.softmax_scale(cfg), cfg["causal"], rows=sample_rows(cfg["N"], 1024), label=name)
 
 
 @pytest.mark.parametrize("B,H,N,d", [(1, 88, 300, 64), (3, 24, 200, 128), (1, 12, 260, 64), (1, 40, 140, 96), (2, 8, 520, 128)])
