@@ -170,6 +170,14 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="cfg3", help="cfg1..cfg5 (cfg3 is the headline)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--schedule", default="auto", choices=["auto", "rolling", "pipelined", "dense"],
+                    help="main loop hint passed to the operator (include/fa8_api.h, FA8_SCHEDULE_*); the results do not depend on it")
+    ap.add_argument("--v-transposed", action="store_true",
+                    help="hand v over as [B,H,d,N], the reference's calling convention (reference test.py:71): the kernel then "
+                         "reads V^T fragments with plain 16-byte LDS reads instead of the transposing ones")
+    ap.add_argument("--inputs", default="workload", choices=["workload", "v-ones", "zeros"],
+                    help="what the timed tensors hold: the workload's own seeded draw; the same with v all ones; all zeros.  "
+                         "Same instructions (zeros: no rescale), fewer toggling bits: shows how far board power sets the clock")
     ap.add_argument("--no-other-workloads", action="store_true",
                     help="skip the kernel times of the other BASELINE workloads (config.other_workloads; headline runs only)")
     ap.add_argument("--settle-seconds", type=float, default=0.25,
@@ -225,11 +233,20 @@ def main():
     q, k, v = q8.to(dev), k8.to(dev), v8.to(dev)
     flops = inputs.flops(cfg)
 
+    if args.inputs == "v-ones":
+        v = torch.ones_like(v, dtype=torch.float32).to(v.dtype)
+    elif args.inputs == "zeros":
+        q, k, v = torch.zeros_like(q), torch.zeros_like(k), torch.zeros_like(v)
+    hint = {"auto": 0, "rolling": 1, "pipelined": 2, "dense": 3}[args.schedule]
+    if args.v_transposed:
+        v = v.transpose(2, 3).contiguous()
+
     def step():
-        return ext.flash_attention_v2_cutlass(q, k, v, causal, scale)[0]
+        return ext.flash_attention_v2_cutlass(q, k, v, causal, scale, v_transposed=args.v_transposed, schedule=hint)[0]
 
     # which of the kernel's main loops the library runs for this launch (include/fa8_api.h, FA8_SCHEDULE_*)
-    plan = fa.lib().fa8_fwd_schedule(ctypes.byref(fa.make_params(q, k, v, step(), causal, scale)))
+    plan = fa.lib().fa8_fwd_schedule(ctypes.byref(fa.make_params(q, k, v, step(), causal, scale, v_transposed=args.v_transposed,
+                                                                 schedule=hint)))
     main_loop = MAIN_LOOPS.get(plan, f"error {plan}")
     for _ in range(args.warmup):
         step()
@@ -301,6 +318,8 @@ def main():
             "algorithmic_hbm_gbps": round(alg_bytes / (kern_avg_ms * 1e-3) / 1e9, 1),
             "kv_block": fa.query(fa.FA8_QUERY_KV_BLOCK),
             "main_loop": main_loop,
+            "v_layout": "[B,H,d,N]" if args.v_transposed else "[B,H,N,d]",
+            "inputs": args.inputs,
             "sclk_mhz_under_load": sclk,
             "board_power_w_under_load": power_w,
             "board_power_cap_w": round(power_cap_w) if power_cap_w is not None else None,
@@ -321,12 +340,12 @@ def main():
         },
     }
 
-    if args.workload == "cfg3" and not args.no_other_workloads:
+    if args.workload == "cfg3" and not args.no_other_workloads and not args.v_transposed and hint == 0 and args.inputs == "workload":
         # the other BASELINE workloads in the same process: kernel time, TFLOP/s and algorithmic HBM rate (value, ms_per_step and
         # roofline above stay the headline's)
         out["config"]["other_workloads"] = [time_other_workload(w, ext, fa, inputs, torch) for w in ("cfg2", "cfg4", "cfg5")]
 
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and args.inputs == "workload":
         # The reference's CPU-runnable path (naive attention, reference test.py:25-33) restated in oracle/ and timed
         # on this machine's host cores, on the first heads of the same workload.
         from oracle.naive_attention import naive_attention_cpu

@@ -26,6 +26,7 @@
 #include <atomic>
 #include <cmath>
 #include <cstdint>
+#include <cstdlib>
 #include <type_traits>
 
 #include "fa8_api.h"
@@ -1068,6 +1069,20 @@ int choose_loop(const Fa8FwdParams* p) {
   return small ? FA8_SCHEDULE_PIPELINED : FA8_SCHEDULE_ROLLING;
 }
 
+// Tuning aid for measurements only: FA8_CAUSAL_INTERLEAVE=n in the environment (read once) replaces the number of heads of an
+// XCD that take turns at every q block of a causal launch (see decode_block; the results do not depend on it).  0: unset.
+int env_causal_interleave() {
+  static std::atomic<int> cached{-1};
+  int v = cached.load(std::memory_order_relaxed);
+  if (v < 0) {
+    const char* e = std::getenv("FA8_CAUSAL_INTERLEAVE");
+    v = e ? std::atoi(e) : 0;
+    if (v < 0 || v > 64) v = 0;
+    cached.store(v, std::memory_order_relaxed);
+  }
+  return v;
+}
+
 bool span_ok(long long outer_stride, long long inner_extent) { return outer_stride >= inner_extent; }
 
 }  // namespace
@@ -1144,6 +1159,7 @@ extern "C" int fa8_fwd(const Fa8FwdParams* p, void* hip_stream) {
   a.n_qblocks = (p->seqlen_q + kQBlock - 1) / kQBlock;
   a.bh_total = p->batch * p->heads;
   a.interleave = a.bh_total / 8 < 8 ? (a.bh_total / 8 > 0 ? a.bh_total / 8 : 1) : 8;  // causal launches, see decode_block
+  if (env_causal_interleave() > 0) a.interleave = env_causal_interleave();
   a.scale_log2 = p->softmax_scale * 1.4426950408889634f;
   a.q_bs = p->q_batch_stride; a.q_hs = p->q_head_stride; a.q_rs = p->q_row_stride;
   a.k_bs = p->k_batch_stride; a.k_hs = p->k_head_stride; a.k_rs = p->k_row_stride;

@@ -116,6 +116,10 @@ int fa8_fwd_validate(const Fa8FwdParams* p);
  * device and return without synchronising.  Replaces run_flash_attn_cutlass + the <<<>>> launch
  * (reference csrc/flash_attention.cu:586-637), which uses stream 0 and cudaDeviceSynchronize().
  * The caller keeps q/k/v/o alive until the stream has passed the work.  Stateless and re-entrant.
+ * The current HIP device must be the one that owns the stream and the tensors (the library asks it for its number of
+ * compute units when it chooses the main loop).  The parameter block has grown from version to version and carries no
+ * size field: a caller compares fa8_query(FA8_QUERY_PARAMS_SIZE) with its own sizeof(Fa8FwdParams) once, before the first
+ * call, and zero-initialises the whole block.
  */
 int fa8_fwd(const Fa8FwdParams* p, void* hip_stream);
 
