@@ -454,10 +454,14 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
       float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * c);
       if constexpr (kMasked) alpha = (m_run == -INFINITY) ? 0.f : alpha;
       l_run *= alpha;
+      // only the lanes of the queries whose max moved multiply (the others would multiply by exactly 1): the instructions are
+      // issued either way, but idle lanes draw no power, and this kernel runs at the board's power limit
+      if (alpha != 1.f) {
 #pragma unroll
-      for (int mt = 0; mt < kMTiles; ++mt)
+        for (int mt = 0; mt < kMTiles; ++mt)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) o_acc[mt][i] *= alpha;
+          for (int i = 0; i < 16; ++i) o_acc[mt][i] *= alpha;
+      }
       m_run = m_new;
     }
     float mc = m_new * c;
@@ -611,12 +615,14 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
       }
       l_run += sum0 + sum1;
       asm volatile("" : "+v"(l_run));  // keeps the additions above where they are written
-      // O now holds the PV product of block j-1: bring it to the new row max
+      // O now holds the PV product of block j-1: bring it to the new row max (in the lanes whose max moved, see compute_tile)
       if (changed) {
+        if (alpha != 1.f) {
 #pragma unroll
-        for (int mt = 0; mt < kMTiles; ++mt)
+          for (int mt = 0; mt < kMTiles; ++mt)
 #pragma unroll
-          for (int i = 0; i < 16; ++i) o_acc[mt][i] *= alpha;
+            for (int i = 0; i < 16; ++i) o_acc[mt][i] *= alpha;
+        }
       }
       p8 = p8_cur;
     };
@@ -775,12 +781,15 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
       }
       l_run += sum0 + sum1;
       asm volatile("" : "+v"(l_run));  // keeps the additions above where they are written (sunk to the end they cost registers)
-      // O now holds the PV product of block j-1 (issued four or more chunks ago): bring it to the new row max
+      // O now holds the PV product of block j-1 (issued four or more chunks ago): bring it to the new row max (in the lanes
+      // whose max moved, see compute_tile)
       if (changed) {
+        if (alpha != 1.f) {
 #pragma unroll
-        for (int mt = 0; mt < kMTiles; ++mt)
+          for (int mt = 0; mt < kMTiles; ++mt)
 #pragma unroll
-          for (int i = 0; i < 16; ++i) o_acc[mt][i] *= alpha;
+            for (int i = 0; i < 16; ++i) o_acc[mt][i] *= alpha;
+        }
       }
     };
     // Every step starts two tile copies, also past the last block this workgroup walks (those copy nothing, see issue_k), so the
