@@ -25,7 +25,7 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch of the headline workload read by rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), each scaled by
 # what the same counter reads for a plain copy kernel of known size; see profiles/.  None until measured.
 MEASURED_TRAFFIC_BYTES = {"cfg3": 168.0e6,  # profiles/fa8_fwd_kernel_d128_cfg3_headline.md, section 3
-                          "cfg2": 21.30e6, "cfg4": 368.6e6, "cfg5": 105.5e6}  # profiles/fa8_fwd_kernel_cfg2_cfg4_cfg5.md
+                          "cfg2": 21.12e6, "cfg4": 364.2e6, "cfg5": 104.2e6}  # profiles/fa8_fwd_kernel_cfg2_cfg4_cfg5.md
 
 
 TRAFFIC_SOURCE = {"cfg3": "profiles/fa8_fwd_kernel_d128_cfg3_headline.md", "cfg2": "profiles/fa8_fwd_kernel_cfg2_cfg4_cfg5.md",
