@@ -124,6 +124,47 @@ def read_power_w():
     return now, first(base + "power1_cap")
 
 
+def measure_traffic(workload):
+    """HBM bytes per launch of one workload, measured now: four rocprofv3 --pmc child runs of this script (FETCH_SIZE and
+    WRITE_SIZE, each for the kernel and for a plain 256 MiB device copy that gives the counter's scale).  This process must not
+    have touched the GPU yet (it only starts children).  Prints one JSON line."""
+    import csv
+    import glob
+    import shutil
+    import subprocess
+    import tempfile
+    rocprof = shutil.which("rocprofv3") or os.path.join(os.environ.get("ROCM_PATH", "/opt/rocm"), "bin", "rocprofv3")
+    tmp = tempfile.mkdtemp(prefix="fa8_traffic_", dir=os.environ.get("TMPDIR", "/tmp"))
+
+    def counter(name, args, kernel_substr):
+        out = os.path.join(tmp, name + "_" + str(len(os.listdir(tmp))))
+        cmd = [rocprof, "--pmc", name, "--output-format", "csv", "-d", out, "--", sys.executable, os.path.abspath(__file__)] + args
+        subprocess.run(cmd, check=True, cwd=tmp, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL, timeout=170)
+        vals = []
+        for f in glob.glob(os.path.join(out, "**", "*_counter_collection.csv"), recursive=True):
+            with open(f) as fh:
+                vals += [float(r["Counter_Value"]) for r in csv.DictReader(fh)
+                         if kernel_substr in r["Kernel_Name"] and r["Counter_Name"] == name]
+        if not vals:
+            raise RuntimeError(f"no {name} rows for {kernel_substr}")
+        return sum(vals) / len(vals), len(vals)
+    kern_args = ["--workload", workload, "--no-cpu-baseline", "--no-other-workloads", "--steps", "5", "--warmup", "2",
+                 "--settle-seconds", "0"]
+    copy_kib = float(256 << 10)
+    res = {}
+    for name in ("FETCH_SIZE", "WRITE_SIZE"):
+        cal, _ = counter(name, ["--copy-calibration"], "copyBuffer")
+        kib, n = counter(name, kern_args, "fa8_fwd_kernel")
+        res[name] = {"kib_per_launch": round(kib, 1), "launches": n, "copy_256MiB_reads": round(cal, 1),
+                     "scale": round(copy_kib / cal, 3), "bytes_per_launch": kib * 1024.0 * copy_kib / cal}
+    shutil.rmtree(tmp, ignore_errors=True)
+    from cutlass_flash_atten_fp8_amd import inputs
+    alg = inputs.algorithmic_bytes(inputs.CONFIGS[workload])
+    total = res["FETCH_SIZE"]["bytes_per_launch"] + res["WRITE_SIZE"]["bytes_per_launch"]
+    print(json.dumps({"workload": workload, "hbm_bytes_per_launch": round(total), "algorithmic_bytes": alg,
+                      "traffic_ratio": round(total / alg, 3), "counters": res}), flush=True)
+
+
 def time_other_workload(name, ext, fa, inputs, torch, launches=20, settle_seconds=0.15):
     """Kernel time of one more BASELINE workload, measured like the headline: clock-settle launches, then one HIP-event pair
     per launch on torch's current stream.  Returns the entry of config.other_workloads."""
@@ -191,6 +232,9 @@ def main():
                     help="run only the instruction-mix probe (bench_mix_probe.hip beside this file, built with hipcc on first "
                          "use): what a SIMD needs for the vector and matrix instructions of one KV block, then with the LDS "
                          "operand reads, the tile copies and the barrier of the loop added; prints its JSON lines")
+    ap.add_argument("--measure-traffic", action="store_true",
+                    help="measure the HBM bytes per launch of --workload now: runs rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on "
+                         "child runs of this script and of its --copy-calibration (the figure roofline.traffic quotes)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a plain 256 MiB device-to-device copy (10 times): the known-size kernel that the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run are scaled by")
@@ -200,6 +244,9 @@ def main():
               "range of heads and run this same kernel, with no communication); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
 
+    if args.measure_traffic:
+        measure_traffic(args.workload)
+        return
     if args.instruction_mix:
         import subprocess
         src, exe = os.path.join(ROOT, "bench_mix_probe.hip"), os.path.join(ROOT, "bench_mix_probe")
