@@ -388,7 +388,11 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
   for (int mt = 0; mt < kMTiles; ++mt)
 #pragma unroll
     for (int i = 0; i < 16; ++i) o_acc[mt][i] = 0.f;
-  float m_run = -INFINITY;  // running row max of raw S (both half-lanes of a query hold the same value)
+  // running row max of raw S (both half-lanes of a query hold the same value).  The pipelined loop starts it at a finite value
+  // below every possible logit (|s| <= 57344^2 * 256 < 1e12) instead of -inf: a row that has not seen a key yet then needs no
+  // special case (its rescale factor exp2((m_run - m_new) * c) is 0 or multiplies zeros, m_new * c stays finite, and a masked
+  // logit -inf still gives exp2(-inf) = 0 for the positive scales this loop runs with); the results are the same bit for bit.
+  float m_run = PIPE ? -1.0e30f : -INFINITY;
   float l_run = 0.f;        // this lane's share of the running row sum
 
   // K fragment of S^T sub-tile t, k-step ks, and V^T fragment of O^T tile mt, from the tiles in kb / vb
@@ -727,12 +731,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FA8_WA
         changed = __any(m_new != m_run);
         if (changed) {
           alpha = __builtin_amdgcn_exp2f((m_run - m_new) * c);
-          if (masked) alpha = (m_run == -INFINITY) ? 0.f : alpha;  // a row that has not seen a key yet
           l_run *= alpha;
           m_run = m_new;
         }
       }
-      if (masked) mc = (m_new == -INFINITY) ? 0.f : mc;
       float sum0, sum1;
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -1055,8 +1057,9 @@ int compute_units() {
 }
 
 // Which main loop a valid call runs (see fa8_fwd_kernel): FA8_SCHEDULE_ROLLING, _PIPELINED or _DENSE.
-// The pipelined loops exist for head dims 64 and 128 and for a positive softmax scale (the pipelined loop relies on
-// exp2(-inf * scale) = 0 for masked logits); elsewhere every hint is ignored and the rolling loop runs.
+// The pipelined loops exist for head dims 64 and 128 and for a softmax scale in (0, 1e6) (the pipelined loop relies on
+// exp2(-inf * scale) = 0 for masked logits and on its finite stand-in for a row max of -inf times the scale staying finite);
+// elsewhere every hint is ignored and the rolling loop runs.
 // Dense: full (non-causal) attention over a whole number of KV blocks, where no logit is ever masked; measured 1 - 2 % faster
 // than the rolling loop on launches that fill the chip and 3 - 5 % faster than the pipelined loop on small ones, so it is
 // the choice wherever it applies.  A hint for it that does not apply falls back to the automatic choice.
@@ -1065,7 +1068,7 @@ int compute_units() {
 // causal launches the thinning out of the workgroups, is a large share of the run).  Measured 5 - 15 % faster than the
 // rolling loop there; the rolling loop is equal or up to 5 % faster elsewhere.
 int choose_loop(const Fa8FwdParams* p) {
-  if ((p->head_dim != 64 && p->head_dim != 128) || !(p->softmax_scale > 0.f)) return FA8_SCHEDULE_ROLLING;
+  if ((p->head_dim != 64 && p->head_dim != 128) || !(p->softmax_scale > 0.f && p->softmax_scale < 1.0e6f)) return FA8_SCHEDULE_ROLLING;
   const bool dense_ok = !p->is_causal && p->seqlen_k % kKvBlock == 0;
   if (p->schedule == FA8_SCHEDULE_ROLLING || p->schedule == FA8_SCHEDULE_PIPELINED) return p->schedule;
   if (dense_ok) return FA8_SCHEDULE_DENSE;

@@ -44,7 +44,7 @@ extern "C" {
  *   PIPELINED software-pipelined over neighbouring KV blocks, two wavefronts per SIMD: for small masked launches
  *   DENSE     the same pipeline in three wavefronts per SIMD, for launches without any masked logit: full (non-causal)
  *             attention with seqlen_k a multiple of 64; asked for elsewhere, the library chooses as for AUTO
- *   (PIPELINED and DENSE are built for head dims 64 and 128 and a positive softmax scale; ignored elsewhere) */
+ *   (PIPELINED and DENSE are built for head dims 64 and 128 and a softmax scale in (0, 1e6); ignored elsewhere) */
 #define FA8_SCHEDULE_AUTO 0
 #define FA8_SCHEDULE_ROLLING 1
 #define FA8_SCHEDULE_PIPELINED 2
