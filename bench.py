@@ -88,6 +88,41 @@ def reference_sweep(ext, torch):
                       "inputs N(0,0.5) clamped to +-0.1 (reference test.py:13-23,56-57)", "rows": rows}), flush=True)
 
 
+def shape_sweep(ext, fa, torch):
+    """Kernel time over a grid of shapes at a fixed token count (B*H*N = 262144, the headline's): head dims 64 / 128 / 256,
+    N from 1024 to 16384, full and causal; N(0,1) inputs, scale 1/sqrt(d); 40 event-timed launches per shape after a short
+    settle phase.  One JSON line."""
+    import math
+    rows = []
+    for d in (64, 128, 256):
+        for n, bsz, heads in ((1024, 8, 32), (2048, 4, 32), (4096, 2, 32), (8192, 1, 32), (16384, 1, 16)):
+            g = torch.Generator(device="cpu").manual_seed(7)
+            q, k, v = (torch.randn((bsz, heads, n, d), generator=g).to(torch.float8_e4m3fn).cuda() for _ in range(3))
+            for causal in (False, True):
+                scale = 1.0 / math.sqrt(d)
+                plan = fa.lib().fa8_fwd_schedule(ctypes.byref(fa.make_params(
+                    q, k, v, ext.flash_attention_v2_cutlass(q, k, v, causal, scale)[0], causal, scale)))
+                t0 = time.perf_counter()
+                while time.perf_counter() - t0 < 0.1:
+                    for _ in range(10):
+                        ext.flash_attention_v2_cutlass(q, k, v, causal, scale)
+                    torch.cuda.synchronize()
+                evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(40)]
+                for e0, e1 in evs:
+                    e0.record()
+                    ext.flash_attention_v2_cutlass(q, k, v, causal, scale)
+                    e1.record()
+                torch.cuda.synchronize()
+                ms = sorted(e0.elapsed_time(e1) for e0, e1 in evs)
+                avg = sum(ms) / len(ms)
+                flops = 4.0 * bsz * heads * n * n * d * (0.5 if causal else 1.0)
+                rows.append({"batch": bsz, "heads": heads, "seq_len": n, "head_dim": d, "causal": causal,
+                             "main_loop": MAIN_LOOPS.get(plan, str(plan)), "kernel_ms_avg": round(avg, 5),
+                             "tflops": round(flops / (avg * 1e-3) / 1e12, 1),
+                             "pct_fp8_mfma_peak": round(100.0 * flops / (avg * 1e-3) / 1e12 / FP8_MFMA_PEAK_TFLOPS, 2)})
+    print(json.dumps({"metric": "fp8_attention_fwd_shape_sweep", "unit": "TFLOP/s", "rows": rows}), flush=True)
+
+
 def read_sclk_mhz():
     """Current shader clock from the amdgpu sysfs node (the level marked '*' in pp_dpm_sclk), or None."""
     import glob
@@ -228,6 +263,9 @@ def main():
                     help="instead of the headline step, time the 18 shapes of the reference's own benchmark table "
                          "(reference test.py:95-100: B=1, causal, scale=1/sqrt(N), inputs clamped to +-0.1) and print "
                          "one JSON line holding the table next to the reference's published Ada numbers")
+    ap.add_argument("--shape-sweep", action="store_true",
+                    help="instead of the headline step, time a grid of shapes at the headline's token count (head dims 64, 128, "
+                         "256; N 1024 ... 16384; full and causal) and print one JSON line")
     ap.add_argument("--instruction-mix", action="store_true",
                     help="run only the instruction-mix probe (bench_mix_probe.hip beside this file, built with hipcc on first "
                          "use): what a SIMD needs for the vector and matrix instructions of one KV block, then with the LDS "
@@ -271,6 +309,9 @@ def main():
     ext = fa.load_extension()  # raises if the native code has not been built: there is no fallback path
     if args.reference_sweep:
         reference_sweep(ext, torch)
+        return
+    if args.shape_sweep:
+        shape_sweep(ext, fa, torch)
         return
     cfg = inputs.CONFIGS[args.workload]
     scale = inputs.softmax_scale(cfg)
