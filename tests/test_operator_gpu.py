@@ -243,3 +243,36 @@ def test_capturable_in_a_hip_graph(schedule, causal):
         # eager work and new inputs between replays: the graph reads q/k/v in place
         q.copy_(rand_fp8((2, 4, 384, 128), 60 + i).to(DEV))
         eager = ext.flash_attention_v2_cutlass(q, k, v, causal, 0.09, schedule=schedule)[0].clone()
+
+
+@pytest.mark.parametrize("nk,causal,schedule", [(99968, False, fa.FA8_SCHEDULE_AUTO), (100000, False, fa.FA8_SCHEDULE_PIPELINED),
+                                                (100000, True, fa.FA8_SCHEDULE_ROLLING), (100000, True, fa.FA8_SCHEDULE_PIPELINED)])
+def test_long_kv_with_rows_far_apart(nk, causal, schedule):
+    """100 000 keys whose rows lie 20 480 bytes apart: the kernel's 32-bit byte offsets into k and v run up to 2.05e9, just
+    under the 2^31 the library accepts.  The gaps between the rows hold NaN codes, so a misplaced read shows.  Bit for bit the
+    result of the same call on contiguous copies, and a few rows against the oracle."""
+    d, nq, stride = 128, 200, 20480
+    q, k, v = (rand_fp8((1, 1, n, d), s).to(DEV) for n, s in ((nq, 31), (nk, 32), (nk, 33)))
+    wide = []
+    for t in (k, v):
+        big = torch.full((nk, stride), 0x7F, dtype=torch.uint8, device=DEV)
+        big[:, :d] = t.view(torch.uint8)[0, 0]
+        wide.append(big[:, :d].view(torch.float8_e4m3fn)[None, None])
+    kw, vw = wide
+    assert kw.stride(2) == stride and kw.shape == k.shape
+    scale = 1.0 / math.sqrt(d)
+    outs = []
+    for kk, vv in ((kw, vw), (k, v)):
+        o = torch.empty((1, 1, nq, d), dtype=torch.float16, device=DEV)
+        p = fa.make_params(q, kk, vv, o, causal, scale, causal_bottom_right=True, schedule=schedule)
+        rc = fa.lib().fa8_fwd(ctypes.byref(p), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+        assert rc == 0, fa.error_string(rc)
+        outs.append(o)
+    torch.cuda.synchronize()
+    assert torch.isfinite(outs[0]).all()
+    assert torch.equal(outs[0], outs[1])
+    rows = np.array([0, 1, 63, 64, 127, 128, nq - 1], dtype=np.int32)
+    want = fo.forward(u8(q), u8(k), u8(v), scale, causal=causal, rows=rows, exp2_form=True, causal_bottom_right=True,
+                      matmul_model=fo.MATMUL_GFX950).astype(np.float32)
+    got = outs[0].float().cpu().numpy()[:, :, rows]
+    assert np.abs(got - want).max() <= 2e-2 and np.abs(got - want).mean() <= 2e-3  # the parity bar
