@@ -47,6 +47,39 @@ def test_query_values():
     assert fa.error_string(-999)
 
 
+@pytest.mark.skipif(__import__("shutil").which("gcc") is None, reason="no C compiler")
+def test_header_is_plain_c_and_the_ctypes_mirror_has_its_layout(tmp_path):
+    """include/fa8_api.h compiles as strict C99 on its own, and every field of Fa8FwdParams sits where the ctypes mirror
+    puts it (offset and size, taken from a C program built against the header), as do the numeric codes."""
+    import subprocess
+    fields = [name for name, _ in fa.Fa8FwdParams._fields_]
+    codes = ["FA8_DTYPE_E4M3", "FA8_DTYPE_E5M2", "FA8_OUT_FP16", "FA8_OUT_E4M3", "FA8_OUT_E5M2", "FA8_V_ROWS", "FA8_V_TRANSPOSED",
+             "FA8_CAUSAL_TOP_LEFT", "FA8_CAUSAL_BOTTOM_RIGHT", "FA8_SCHEDULE_AUTO", "FA8_SCHEDULE_ROLLING",
+             "FA8_SCHEDULE_PIPELINED", "FA8_SCHEDULE_DENSE", "FA8_QUERY_VERSION", "FA8_QUERY_KV_BLOCK", "FA8_QUERY_Q_BLOCK",
+             "FA8_QUERY_KV_ASCENDING", "FA8_QUERY_THREADS", "FA8_QUERY_PARAMS_SIZE"]
+    src = tmp_path / "layout.c"
+    lines = ['#include "fa8_api.h"', "#include <stddef.h>", "#include <stdio.h>", "int main(void) {",
+             '  printf("sizeof %zu\\n", sizeof(Fa8FwdParams));']
+    for f in fields:
+        lines.append(f'  printf("{f} %zu %zu\\n", offsetof(Fa8FwdParams, {f}), sizeof(((Fa8FwdParams*)0)->{f}));')
+    for c in codes:
+        lines.append(f'  printf("{c} %d\\n", (int){c});')
+    lines += ["  return 0;", "}"]
+    src.write_text("\n".join(lines) + "\n")
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-std=c99", "-pedantic", "-Wall", "-Wextra", "-Werror", "-I", os.path.join(ROOT, "include"), str(src),
+                    "-o", str(exe)], check=True, capture_output=True)
+    out = dict((ln.split()[0], [int(x) for x in ln.split()[1:]]) for ln in
+               subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.splitlines())
+    assert out["sizeof"] == [ctypes.sizeof(fa.Fa8FwdParams)]
+    for f in fields:
+        d = getattr(fa.Fa8FwdParams, f)
+        assert out[f] == [d.offset, d.size], f
+    assert len(out) == 1 + len(fields) + len(codes)
+    for c in codes:
+        assert out[c] == [getattr(fa, c)], c
+
+
 def cpu_tensors(n=64, d=64, dtype=torch.float8_e4m3fn, b=1, h=2):
     q = torch.zeros((b, h, n, d), dtype=torch.float32).to(dtype)
     return q, q.clone(), q.clone(), torch.zeros((b, h, n, d), dtype=torch.float16)
