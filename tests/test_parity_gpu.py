@@ -108,3 +108,32 @@ def test_every_head_and_q_block_is_computed(B, H, N, d, causal):
     rows = sample_rows(N, 24, seed=H)
     assert_parity(o.float().cpu().numpy()[:, :, rows, :], u8(q), u8(k), u8(v), d ** -0.5, causal=causal, rows=rows,
                   kv_block=fa.query(fa.FA8_QUERY_KV_BLOCK), label=f"map B{B} H{H} N{N} d{d} causal={causal}")
+
+
+@pytest.mark.parametrize("name,chunk", [("cfg3", 512), ("cfg4", 1024), ("cfg5", 2000)])
+def test_full_size_rows_do_not_depend_on_the_launch(name, chunk):
+    """Every row of the full-size workloads, not only the rows sampled for the oracle: a query row's result depends on its
+    own q row and on the keys it sees, not on the launch it is part of.  The full launch (NaN-filled output first: every row
+    must be written, twice the same bits) is compared bit for bit with launches of `chunk` query rows at a time over the same
+    keys (causal: the keys up to the chunk's last row, diagonal aligned bottom right), which map workgroups to heads, q blocks and
+    XCDs differently and mostly take another main loop."""
+    cfg = inputs.CONFIGS[name]
+    dev = torch.device("cuda:0")
+    q, k, v = (t.to(dev) for t in inputs.make_qkv(cfg))
+    scale, causal, N = inputs.softmax_scale(cfg), cfg["causal"], cfg["N"]
+    full = torch.full(q.shape, float("nan"), dtype=torch.float16, device=dev)
+    run_abi(q, k, v, causal, scale, o=full)
+    assert torch.isfinite(full).all()
+    again = run_abi(q, k, v, causal, scale)
+    assert torch.equal(full, again)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for r0 in range(0, N, chunk):
+        r1 = min(N, r0 + chunk)
+        qc = q[:, :, r0:r1]
+        kc, vc = (k[:, :, :r1], v[:, :, :r1]) if causal else (k, v)
+        o = torch.empty((cfg["B"], cfg["H"], r1 - r0, cfg["d"]), dtype=torch.float16, device=dev)
+        p = fa.make_params(qc, kc, vc, o, causal, scale, causal_bottom_right=True)
+        rc = fa.lib().fa8_fwd(ctypes.byref(p), stream)
+        assert rc == 0, fa.error_string(rc)
+        torch.cuda.synchronize()
+        assert torch.equal(o, full[:, :, r0:r1]), (name, r0)
