@@ -124,6 +124,74 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WIDE ? 2 : 
   }
 }
 
+
+// The matrix pipe alone: every wavefront issues v_mfma_f32_32x32x64_f8f6f4 back to back (four accumulators, four A and four B
+// fragments in registers, three wavefronts per SIMD), once on constant operands and once on operands that differ from lane to lane
+// and from instruction to instruction (e4m3 codes of random sign and mantissa with exponents spread over five binades, the spread
+// of N(0,1) draws): what the board delivers under its power limit when nothing but the matrix pipe works.
+template <int RANDOM>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3))) void mfma_alone_kernel(float* out, int iters, long long* clk) {
+  v8i a[4], b[4];
+  unsigned x = (blockIdx.x * 256u + threadIdx.x) * 2654435761u + 12345u;
+  for (int f = 0; f < 4; ++f)
+    for (int i = 0; i < 8; ++i) {
+      unsigned wa = 0, wb = 0;
+      for (int byte = 0; byte < 4; ++byte) {
+        x ^= x << 13, x ^= x >> 17, x ^= x << 5;
+        const unsigned ca = RANDOM ? ((x & 0x80u) | ((4u + (x >> 8) % 5u) << 3) | ((x >> 16) & 7u)) : 0x38u;   // 0x38 = 1.0
+        const unsigned cb = RANDOM ? (((x >> 1) & 0x80u) | ((4u + (x >> 12) % 5u) << 3) | ((x >> 20) & 7u)) : 0x38u;
+        wa |= ca << (8 * byte);
+        wb |= cb << (8 * byte);
+      }
+      a[f][i] = (int)wa;
+      b[f][i] = (int)wb;
+    }
+  v16f acc[4];
+  for (int t = 0; t < 4; ++t)
+    for (int i = 0; i < 16; ++i) acc[t][i] = 0.f;
+  const long long t0 = clock64();
+  const long long w0 = wall_clock64();
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int g = 0; g < 8; ++g)
+      acc[g & 3] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[g & 3], b[(g + (g >> 2)) & 3], acc[g & 3], 0, 0, 0, 0, 0, 0);
+  }
+  const long long t1 = clock64();
+  const long long w1 = wall_clock64();
+  float s = 0;
+  for (int t = 0; t < 4; ++t)
+    for (int i = 0; i < 16; ++i) s += acc[t][i];
+  if (s == 1.2345f) out[0] = s;
+  if (blockIdx.x == 100 && threadIdx.x == 0) {
+    clk[0] = t1 - t0;
+    clk[1] = w1 - w0;
+  }
+}
+
+template <int RANDOM>
+int run_mfma_alone(const char* name, float* dout, long long* dclk) {
+  const int iters = 40000, grid = 768;
+  float ms = 0;
+  long long hclk[2] = {0, 1};
+  for (int rep = 0; rep < 3; ++rep) {  // the last of three launches: the clock has settled under the load by then
+    hipEvent_t e0, e1;
+    CK(hipEventCreate(&e0));
+    CK(hipEventCreate(&e1));
+    CK(hipEventRecord(e0));
+    hipLaunchKernelGGL((mfma_alone_kernel<RANDOM>), dim3(grid), dim3(256), 0, 0, dout, iters, dclk);
+    CK(hipEventRecord(e1));
+    CK(hipEventSynchronize(e1));
+    CK(hipEventElapsedTime(&ms, e0, e1));
+    CK(hipMemcpy(hclk, dclk, 16, hipMemcpyDeviceToHost));
+  }
+  const double flop = (double)grid * 4 * iters * 8 * 2.0 * 32 * 32 * 64;
+  const double ghz = (double)hclk[0] / ((double)hclk[1] * 10.0);
+  printf("{\"mix\": \"%s\", \"wavefronts_per_simd\": 3, \"launch_ms\": %.2f, \"tflops\": %.0f, \"sclk_ghz\": %.2f, "
+         "\"pct_of_5_pflops\": %.1f}\n", name, ms, flop / (ms * 1e-3) / 1e12, ghz, flop / (ms * 1e-3) / 5.0e15 * 100);
+  fflush(stdout);
+  return 0;
+}
+
 template <int FLAGS, int WIDE>
 int run(const char* name, float* dout, const uint8_t* src, long long* dclk) {
   const int iters = 3000;
@@ -172,5 +240,7 @@ int main() {
   run<kValu | kMfma, 1>("wide: vector + matrix", dout, src, dclk);
   run<kValu | kMfma | kLdsReads | kCopies | kBarrier, 1>("wide: everything, V^T fragments shared", dout, src, dclk);
   run<kValu | kMfma | kLdsReads | kCopies | kBarrier, 2>("wide: everything, no fragment shared", dout, src, dclk);
+  run_mfma_alone<0>("matrix pipe alone, constant operands", dout, dclk);
+  run_mfma_alone<1>("matrix pipe alone, random operands", dout, dclk);
   return 0;
 }
